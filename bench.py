@@ -1,0 +1,216 @@
+#!/usr/bin/env python3
+"""Benchmark of the Helix all-to-all loopback on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--channels N]
+
+One step = one loopback exchange of all cp logical ranks of the workload
+(payload read + FIFO write + FIFO read + output write), inputs resident in HBM.
+Prints ONE JSON line: effective GB/s (algorithmic bytes / time per call) and
+microseconds per call, the roofline fraction of the exchange kernel (measured
+with HIP events on the launch stream) and a CPU baseline (the reference tests'
+torch transpose recipe and the C restatement of the reference kernel, timed on
+this machine's host cores).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for _p in (ROOT / "helix-a2a_amd", ROOT, ROOT / "tests"):
+    if str(_p) not in sys.path:
+        sys.path.insert(0, str(_p))
+
+METRIC = "µs/call + effective HBM GB/s (% of peak) for Helix a2a, cp=4/8, 1 GPU"
+PEAK_HBM_GBPS = 8000.0
+
+# HBM traffic per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE runs, scaled by
+# the same counters of a plain copy kernel); keyed by (workload, channel count used). Filled in from
+# the summaries under profiles/ when they exist for the configuration that is being run.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def percentile(sorted_vals, q):
+    if not sorted_vals:
+        return None
+    i = min(len(sorted_vals) - 1, max(0, int(round(q * (len(sorted_vals) - 1)))))
+    return sorted_vals[i]
+
+
+def cpu_baseline(w, budget_s: float = 12.0):
+    """Time the CPU restatements on this host for the same workload (bounded sample)."""
+    import torch
+
+    from helix_a2a.workloads import make_inputs
+    from helix_testing import torch_bits
+    from oracle import helix_oracle as ho
+
+    ins_o, ins_s = make_inputs(w, "cpu")
+    threads = torch.get_num_threads()
+    # 1) the reference tests' recipe: transpose, equal-split hand-off, transpose (tests/test_alltoall.py:274-297)
+    for _ in range(2):
+        ho.exchange_transpose_style(ins_o)
+        ho.exchange_transpose_style(ins_s)
+    times = []
+    t_end = time.perf_counter() + budget_s * 0.6
+    while len(times) < 200 and (len(times) < 20 or time.perf_counter() < t_end):
+        t0 = time.perf_counter()
+        ho.exchange_transpose_style(ins_o)
+        ho.exchange_transpose_style(ins_s)
+        times.append(time.perf_counter() - t0)
+        if len(times) >= 20 and time.perf_counter() > t_end:
+            break
+    times.sort()
+    p50 = percentile(times, 0.5)
+    # 2) the C restatement of the reference kernel (its FIFO + LL128 algorithm), one thread, a few calls
+    model = ho.RefModel()
+    sm = 16
+    ws = model.new_workspace(w.cp, sm)
+    for r in range(w.cp):
+        model.init_workspace(ws, r, w.cp, sm)
+    np_o, np_s = [torch_bits(t) for t in ins_o], [torch_bits(t) for t in ins_s]
+    model_times = []
+    t_end = time.perf_counter() + budget_s * 0.4
+    while len(model_times) < 3 or (time.perf_counter() < t_end and len(model_times) < 20):
+        t0 = time.perf_counter()
+        model.alltoall_all_ranks(np_o, np_s, ws, sm_count=sm)
+        model_times.append(time.perf_counter() - t0)
+    model_times.sort()
+    m50 = percentile(model_times, 0.5)
+    return {
+        "value": w.exchange_bytes / p50 / 1e9,
+        "unit": "GB/s",
+        "us_per_call": p50 * 1e6,
+        "cores": threads,
+        "host_cpus": os.cpu_count(),
+        "kind": "port",
+        "sample": (f"{len(times)} calls of the torch-CPU transpose/hand-off/transpose exchange of workload {w.name} "
+                   f"(all {w.cp} ranks, bf16+fp32), p50; GB/s uses the GPU path's algorithmic bytes so the ratio "
+                   f"is a time ratio"),
+        "reference_kernel_model": {
+            "us_per_call": m50 * 1e6,
+            "cores": 1,
+            "sample": f"{len(model_times)} calls of the sequential C restatement of the reference FIFO/LL128 kernel, p50",
+        },
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--workload", default="c3")
+    ap.add_argument("--channels", type=int, default=0, help="0 = automatic")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-check", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs all context-parallel ranks as logical ranks of ONE GPU; "
+              "--gpus must be 1 (nothing here uses a second device)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import helix_a2a
+    from helix_a2a import _ops
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from oracle import helix_oracle as ho
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    torch.cuda.set_device(0)
+    w = WORKLOADS[args.workload]
+    ws = helix_a2a.allocate_workspace(w.cp, 0)
+    for r in range(w.cp):
+        helix_a2a.init_workspace(ws, r, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    plan = _ops.LoopbackPlan(ins_o, ins_s, ws, args.channels)
+    channels = args.channels or _ops.auto_channel_count(w.cp, w.tokens)
+
+    for _ in range(args.warmup):
+        plan.run()
+    torch.cuda.synchronize()
+
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        starts[i].record()
+        plan.run()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    status = _ops.device_status()
+
+    kernel_ms = sorted(s.elapsed_time(e) for s, e in zip(starts, ends))
+    avg_kernel_ms = statistics.fmean(kernel_ms)
+    ms_per_step = wall * 1e3 / args.steps
+    bytes_per_call = w.exchange_bytes
+
+    ok = status == 0
+    if not args.no_check:
+        outs_o, outs_s = plan.run()
+        torch.cuda.synchronize()
+        want_o, want_s = ho.exchange_single_copy(ins_o), ho.exchange_single_copy(ins_s)
+        for r in range(w.cp):
+            ok &= torch.equal(outs_o[r].view(torch.int16), want_o[r].view(torch.int16))
+            ok &= torch.equal(outs_s[r].view(torch.int32), want_s[r].view(torch.int32))
+
+    achieved = bytes_per_call / (avg_kernel_ms * 1e-3) / 1e9
+    result = {
+        "metric": METRIC,
+        "value": bytes_per_call / (ms_per_step * 1e-3) / 1e9,
+        "unit": "GB/s",
+        "us_per_call": ms_per_step * 1e3,
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8",
+        "data": "synthetic",
+        "bit_exact": bool(ok),
+        "config": {
+            "workload": f"{w.name}: Helix a2a loopback, cp={w.cp} logical ranks, T={w.tokens}, H={w.heads}, D={w.head_dim}, "
+                        f"partial_o bf16 [T,cp,H/cp,D] + softmax_stats fp32 [T,cp,H/cp,2], exchange only",
+            "cp": w.cp, "T": w.tokens, "H": w.heads, "D": w.head_dim,
+            "channels": channels,
+            "algorithmic_bytes_per_call": bytes_per_call,
+            "payload_bytes": w.payload_bytes, "wire_bytes": w.wire_bytes,
+        },
+        "kernel_us": {
+            "mean": avg_kernel_ms * 1e3,
+            "p50": percentile(kernel_ms, 0.5) * 1e3,
+            "p5": percentile(kernel_ms, 0.05) * 1e3,
+            "p95": percentile(kernel_ms, 0.95) * 1e3,
+            "min": kernel_ms[0] * 1e3,
+            "max": kernel_ms[-1] * 1e3,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "helix_exchange_kernel",
+            "achieved": achieved,
+            "peak": PEAK_HBM_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / PEAK_HBM_GBPS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, channels)),
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(result))
+    return 0 if ok else 1
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,58 @@
+"""Build libhelix_a2a.so for gfx950 with hipcc.
+
+    python helix-a2a_amd/build.py
+
+Cross-compiles without a GPU. The library is written next to the Python
+package (helix_a2a/libhelix_a2a.so) so that it travels with the source tree.
+This takes the place of the reference's CUDAExtension build (setup.py:14-43).
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from pathlib import Path
+
+HERE = Path(__file__).resolve().parent
+SOURCES = [HERE / "csrc" / "helix_kernels.hip", HERE / "csrc" / "helix_c_api.hip"]
+OUTPUT = HERE / "helix_a2a" / "libhelix_a2a.so"
+
+HIPCC_FLAGS = [
+    "-O3",
+    "-std=c++17",
+    "--offload-arch=gfx950",
+    "-fPIC",
+    "-shared",
+    "-Wall",
+    "-Wno-unused-command-line-argument",
+    # keep the compiler from forming packed-fp32 instructions
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def find_hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and Path(cand).exists():
+            return cand
+    raise RuntimeError("hipcc not found (set HIPCC or install ROCm)")
+
+
+def build_library(verbose: bool = True) -> Path:
+    cmd = [find_hipcc(), *HIPCC_FLAGS, *map(str, SOURCES), "-o", str(OUTPUT)]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "unknown and unsupported"  # host pass does not know the packed-fp32 feature
+    log = "\n".join(l for l in (proc.stdout + proc.stderr).splitlines() if noise not in l)
+    if verbose and log.strip():
+        print(log, flush=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed with exit code {proc.returncode}\n{log}")
+    return OUTPUT
+
+
+if __name__ == "__main__":
+    build_library()
+    print(f"built {OUTPUT}")
+    sys.exit(0)

@@ -1,0 +1,391 @@
+// helix_c_api.hip -- host side of the C ABI declared in include/helix_a2a.h.
+//
+// Validates launch descriptors the way the reference binding validates its
+// tensors (csrc/torch_binding.cpp:40-63,65-129), picks the channel count,
+// splits a call into stream-ordered rounds when one round would overflow the
+// FIFOs, and launches the gfx950 kernels. Errors come back as status codes
+// with a thread-local message; nothing here aborts the process.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+
+#include "../../include/helix_a2a.h"
+#include "helix_kernels.hpp"
+
+namespace {
+
+using namespace helix;
+
+thread_local char g_lastError[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_lastError, sizeof(g_lastError), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define HELIX_HIP_TRY(call)                                                                       \
+  do {                                                                                            \
+    hipError_t err__ = (call);                                                                    \
+    if (err__ != hipSuccess)                                                                      \
+      return fail(HELIX_A2A_ERR_RUNTIME, "%s failed: %s", #call, hipGetErrorString(err__));       \
+  } while (0)
+
+std::atomic<uint64_t> g_spinLimitUs{2000000};
+std::atomic<int> g_singleRound{0};
+
+constexpr int kMaxDevices = 64;
+struct DeviceState {
+  std::once_flag once;
+  hipError_t initError = hipSuccess;
+  int cuCount = 0;
+  uint32_t* status = nullptr;  // device status word
+};
+DeviceState g_devices[kMaxDevices];
+
+// status word: one per device, lives until the process ends
+__device__ uint32_t g_statusWord[4];
+
+int device_state(DeviceState** out) {
+  int dev = 0;
+  HELIX_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(HELIX_A2A_ERR_RUNTIME, "device index %d out of range", dev);
+  DeviceState& st = g_devices[dev];
+  std::call_once(st.once, [&]() {
+    hipDeviceProp_t prop;
+    st.initError = hipGetDeviceProperties(&prop, dev);
+    if (st.initError != hipSuccess) return;
+    st.cuCount = prop.multiProcessorCount;
+    void* p = nullptr;
+    st.initError = hipGetSymbolAddress(&p, HIP_SYMBOL(g_statusWord));
+    if (st.initError != hipSuccess) return;
+    st.status = static_cast<uint32_t*>(p);
+    st.initError = hipMemset(st.status, 0, sizeof(uint32_t) * 4);
+  });
+  if (st.initError != hipSuccess)
+    return fail(HELIX_A2A_ERR_RUNTIME, "device %d setup failed: %s", dev, hipGetErrorString(st.initError));
+  *out = &st;
+  return HELIX_A2A_OK;
+}
+
+int resolve_cu_count(int cuCount, int* out) {
+  if (cuCount < 0) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "cu_count must be >= 0, got %d", cuCount);
+  if (cuCount > 0) {
+    *out = cuCount;
+    return HELIX_A2A_OK;
+  }
+  DeviceState* st = nullptr;
+  int rc = device_state(&st);
+  if (rc != HELIX_A2A_OK) return rc;
+  *out = st->cuCount;
+  return HELIX_A2A_OK;
+}
+
+int check_cp_size(int cpSize) {
+  if (cpSize < 1 || cpSize > kMaxCpSize)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "cp_size must be in [1, %d], got %d", kMaxCpSize, cpSize);
+  return HELIX_A2A_OK;
+}
+
+// One wavefront per (sender, receiver, channel) and direction; aim for one
+// resident wavefront slot per sender stream on a device that holds
+// 32 wavefronts per CU, and never more channels than entries.
+int auto_channels(int cpSize, int entryCount, int cuCount) {
+  int maxCh = max_channel_count(cpSize, cuCount);
+  long slots = static_cast<long>(cuCount) * 32;
+  long c = slots / (static_cast<long>(cpSize) * cpSize);
+  if (c > maxCh) c = maxCh;
+  if (c > entryCount) c = entryCount;
+  if (c < 1) c = 1;
+  return static_cast<int>(c);
+}
+
+int env_channel_count() {
+  // HELIX_A2A_CHANNEL_COUNT as in csrc/torch_binding.cpp:25-32, but re-read on
+  // every call so a sweep can change it without restarting the process.
+  const char* env = std::getenv("HELIX_A2A_CHANNEL_COUNT");
+  if (!env || !*env) return 0;
+  int v = std::atoi(env);
+  return v > 0 ? v : 0;
+}
+
+struct Plan {
+  KernelArgs args;
+  int entryCount;
+  int roundEntries;  // entries per stream-ordered round (multiple of runChannels)
+  MsgShape shape;
+  int cuCount;
+};
+
+int check_field(const helix_a2a_field_t& f, const char* name, int eltSize, int entryCount, int cpSize,
+                bool needData) {
+  if (needData && f.data == nullptr) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%s: data pointer is null", name);
+  if (f.element_size != eltSize)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%s: element size must be %d bytes, got %d", name, eltSize,
+                f.element_size);
+  if (f.element_count <= 0) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%s: element count must be positive", name);
+  long bytes = static_cast<long>(f.element_count) * f.element_size;
+  if (f.stride_bytes < bytes || (f.stride_bytes % kPieceBytes) != 0)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%s: row stride %d must be a multiple of 8 and >= row size %ld", name,
+                f.stride_bytes, bytes);
+  if ((reinterpret_cast<uintptr_t>(f.data) % kPieceBytes) != 0)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%s: data pointer must be 8-byte aligned", name);
+  double extent = static_cast<double>(entryCount) * cpSize * f.stride_bytes;
+  if (extent >= 2147483648.0)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%s: tensor extent %.0f bytes exceeds 2 GiB", name, extent);
+  return HELIX_A2A_OK;
+}
+
+// Validate `count` rank descriptors that share one exchange and build the
+// kernel argument block. `exchangeOutputs` selects whether recv_fields are
+// checked (exchange) or ignored (combine).
+int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs, Plan* plan) {
+  if (ranks == nullptr || count < 1) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "no rank descriptors given");
+  const helix_a2a_params_t& p0 = ranks[0];
+  int rc = check_cp_size(p0.cp_size);
+  if (rc) return rc;
+  const int cp = p0.cp_size;
+  if (count > cp) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%d rank descriptors for cp_size %d", count, cp);
+  if (p0.entry_count < 0) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "entry_count must be >= 0");
+  if (p0.workspace == nullptr) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace pointer is null");
+  if ((reinterpret_cast<uintptr_t>(p0.workspace) % kUnitBytes) != 0 || (p0.workspace_stride_u64 % 2) != 0)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace rows must be 16-byte aligned");
+
+  int cuCount = 0;
+  rc = resolve_cu_count(0, &cuCount);
+  if (rc) return rc;
+  const int maxCh = max_channel_count(cp, cuCount);
+  if (p0.max_channel_count != maxCh)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "max_channel_count %d does not match the device's %d (cp_size %d, %d CUs)",
+                p0.max_channel_count, maxCh, cp, cuCount);
+  if (p0.workspace_stride_u64 * 8ull < workspace_bytes(cp, maxCh))
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace row of %llu bytes is smaller than the %llu bytes cp_size %d needs",
+                static_cast<unsigned long long>(p0.workspace_stride_u64 * 8ull),
+                static_cast<unsigned long long>(workspace_bytes(cp, maxCh)), cp);
+
+  KernelArgs a;
+  std::memset(&a, 0, sizeof(a));
+  bool seen[kMaxCpSize] = {false};
+  for (int i = 0; i < count; ++i) {
+    const helix_a2a_params_t& p = ranks[i];
+    if (p.cp_size != cp || p.entry_count != p0.entry_count || p.workspace != p0.workspace ||
+        p.workspace_stride_u64 != p0.workspace_stride_u64 || p.max_channel_count != p0.max_channel_count ||
+        p.channel_count != p0.channel_count)
+      return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "rank descriptor %d disagrees with descriptor 0", i);
+    if (p.cp_rank < 0 || p.cp_rank >= cp)
+      return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "cp_rank must be in [0, cp_size), got %d", p.cp_rank);
+    if (seen[p.cp_rank]) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "cp_rank %d given twice", p.cp_rank);
+    seen[p.cp_rank] = true;
+    if (p.cp_rank != p0.cp_rank + i)
+      return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "rank descriptors must be consecutive ranks in ascending order");
+    const bool haveData = p.entry_count > 0;
+    if ((rc = check_field(p.send_fields[0], "send partial_o", 2, p.entry_count, cp, haveData))) return rc;
+    if ((rc = check_field(p.send_fields[1], "send softmax_stats", 4, p.entry_count, cp, haveData))) return rc;
+    for (int f = 0; f < 2; ++f) {
+      if (p.send_fields[f].element_count != p0.send_fields[f].element_count ||
+          p.send_fields[f].stride_bytes != p0.send_fields[f].stride_bytes)
+        return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "rank descriptor %d: field %d shape differs from descriptor 0", i, f);
+    }
+    if (exchangeOutputs) {
+      if ((rc = check_field(p.recv_fields[0], "recv partial_o", 2, p.entry_count, cp, haveData))) return rc;
+      if ((rc = check_field(p.recv_fields[1], "recv softmax_stats", 4, p.entry_count, cp, haveData))) return rc;
+      for (int f = 0; f < 2; ++f) {
+        if (p.recv_fields[f].element_count != p0.send_fields[f].element_count ||
+            p.recv_fields[f].stride_bytes != p0.recv_fields[f].stride_bytes)
+          return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "rank descriptor %d: recv field %d shape differs", i, f);
+      }
+    }
+    RankPtrs& rp = a.rank[p.cp_rank];
+    rp.send0 = static_cast<const uint8_t*>(p.send_fields[0].data);
+    rp.send1 = static_cast<const uint8_t*>(p.send_fields[1].data);
+    rp.recv0 = static_cast<uint8_t*>(p.recv_fields[0].data);
+    rp.recv1 = static_cast<uint8_t*>(p.recv_fields[1].data);
+  }
+
+  const int f0 = p0.send_fields[0].element_count * 2;
+  const int f1 = p0.send_fields[1].element_count * 4;
+  // csrc/torch_binding.cpp:95-97,105-106
+  if (f0 % 16 != 0) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "partial_o rows must be a multiple of 16 bytes, got %d", f0);
+  if (p0.send_fields[1].element_count < 2 || p0.send_fields[1].element_count % 2 != 0)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "softmax_stats last dimension must be even and >= 2, got %d",
+                p0.send_fields[1].element_count);
+  MsgShape sh = make_msg_shape(f0, f1);
+  if (sh.lines > kFifoEntryLines)
+    return fail(HELIX_A2A_ERR_CAPACITY, "a message of %d bytes needs %d lines, more than one FIFO entry (%d lines)",
+                f0 + f1, sh.lines, kFifoEntryLines);
+
+  int channels = p0.channel_count > 0 ? p0.channel_count : env_channel_count();
+  if (channels > maxCh)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "channel_count %d exceeds max_channel_count %d", channels, maxCh);
+  if (channels <= 0) channels = auto_channels(cp, p0.entry_count, cuCount);
+
+  DeviceState* st = nullptr;
+  if ((rc = device_state(&st))) return rc;
+
+  a.workspace = reinterpret_cast<uint8_t*>(p0.workspace);
+  a.rowStrideBytes = p0.workspace_stride_u64 * 8ull;
+  a.cpSize = cp;
+  a.maxChannels = maxCh;
+  a.runChannels = channels;
+  a.entryBegin = 0;
+  a.entryEnd = p0.entry_count;
+  a.field0Bytes = f0;
+  a.field1Bytes = f1;
+  a.sendStride0 = p0.send_fields[0].stride_bytes;
+  a.sendStride1 = p0.send_fields[1].stride_bytes;
+  a.recvStride0 = p0.recv_fields[0].stride_bytes;
+  a.recvStride1 = p0.recv_fields[1].stride_bytes;
+  a.rankBegin = p0.cp_rank;
+  a.rankCount = count;
+  a.spinLimitTicks = g_spinLimitUs.load() * 100ull;
+  a.status = st->status;
+
+  plan->args = a;
+  plan->entryCount = p0.entry_count;
+  plan->shape = sh;
+  plan->cuCount = cuCount;
+  // a stream may put 4 entries worth of messages in flight before it needs the receiver
+  long perStream = static_cast<long>(kFifoDepth) * msgs_per_fifo_entry(sh);
+  long roundEntries = perStream * channels;
+  plan->roundEntries = roundEntries > 2000000000L ? 2000000000 : static_cast<int>(roundEntries);
+  return HELIX_A2A_OK;
+}
+
+int launch_rounds(Plan& plan, bool send, bool recv, bool allowRounds, hipStream_t stream) {
+  KernelArgs a = plan.args;
+  a.doSend = send ? 1 : 0;
+  a.doRecv = recv ? 1 : 0;
+  if (plan.entryCount == 0) return HELIX_A2A_OK;
+  const bool fits = plan.entryCount <= plan.roundEntries;
+  if (!fits && !allowRounds)
+    return fail(HELIX_A2A_ERR_CAPACITY,
+                "%d entries over %d channels put more than %d FIFO entries in flight per stream; "
+                "raise the channel count or use the loopback call",
+                plan.entryCount, a.runChannels, kFifoDepth);
+  if (!fits && send && recv && g_singleRound.load()) {
+    // in-kernel back-pressure needs every wavefront of the launch resident
+    long waves = 2L * waves_per_direction(a);
+    if (waves > static_cast<long>(plan.cuCount) * 8)
+      return fail(HELIX_A2A_ERR_CAPACITY, "single-round launch of %ld wavefronts is not guaranteed co-resident", waves);
+    HELIX_HIP_TRY(launch_exchange(a, stream));
+    return HELIX_A2A_OK;
+  }
+  for (int begin = 0; begin < plan.entryCount; begin += plan.roundEntries) {
+    a.entryBegin = begin;
+    long end = static_cast<long>(begin) + plan.roundEntries;
+    a.entryEnd = end > plan.entryCount ? plan.entryCount : static_cast<int>(end);
+    HELIX_HIP_TRY(launch_exchange(a, stream));
+  }
+  return HELIX_A2A_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int helix_a2a_max_channel_count(int cp_size, int cu_count) {
+  if (check_cp_size(cp_size)) return -1;
+  int cu = 0;
+  if (resolve_cu_count(cu_count, &cu)) return -1;
+  return max_channel_count(cp_size, cu);
+}
+
+int64_t helix_a2a_workspace_size_per_rank(int cp_size, int cu_count) {
+  int maxCh = helix_a2a_max_channel_count(cp_size, cu_count);
+  if (maxCh < 0) return -1;
+  return static_cast<int64_t>(workspace_bytes(cp_size, maxCh));
+}
+
+int helix_a2a_auto_channel_count(int cp_size, int entry_count, int cu_count) {
+  if (check_cp_size(cp_size)) return -1;
+  if (entry_count < 0) {
+    fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "entry_count must be >= 0");
+    return -1;
+  }
+  int cu = 0;
+  if (resolve_cu_count(cu_count, &cu)) return -1;
+  return auto_channels(cp_size, entry_count, cu);
+}
+
+int helix_a2a_init_workspace(uint64_t* local_row, int cp_size, int cu_count, void* stream) {
+  int rc = check_cp_size(cp_size);
+  if (rc) return rc;
+  if (local_row == nullptr) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace row pointer is null");
+  if ((reinterpret_cast<uintptr_t>(local_row) % kUnitBytes) != 0)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace row must be 16-byte aligned");
+  int cu = 0;
+  if ((rc = resolve_cu_count(cu_count, &cu))) return rc;
+  int maxCh = max_channel_count(cp_size, cu);
+  HELIX_HIP_TRY(launch_init_row(reinterpret_cast<uint8_t*>(local_row), fifo_region_bytes(cp_size, maxCh),
+                                2 * info_region_bytes(cp_size, maxCh), static_cast<hipStream_t>(stream)));
+  return HELIX_A2A_OK;
+}
+
+int helix_a2a_alltoall(const helix_a2a_params_t* params, void* stream) {
+  Plan plan;
+  int rc = build_plan(params, 1, true, &plan);
+  if (rc) return rc;
+  // both halves in one launch: with peers on the same queue behind this call
+  // the receive half can only time out, so rounds are not an option here
+  return launch_rounds(plan, true, true, plan.args.cpSize == 1, static_cast<hipStream_t>(stream));
+}
+
+int helix_a2a_alltoall_send(const helix_a2a_params_t* per_rank, int rank_count, void* stream) {
+  Plan plan;
+  int rc = build_plan(per_rank, rank_count, true, &plan);
+  if (rc) return rc;
+  return launch_rounds(plan, true, false, false, static_cast<hipStream_t>(stream));
+}
+
+int helix_a2a_alltoall_recv(const helix_a2a_params_t* per_rank, int rank_count, void* stream) {
+  Plan plan;
+  int rc = build_plan(per_rank, rank_count, true, &plan);
+  if (rc) return rc;
+  return launch_rounds(plan, false, true, false, static_cast<hipStream_t>(stream));
+}
+
+int helix_a2a_alltoall_loopback(const helix_a2a_params_t* per_rank, int cp_size, void* stream) {
+  if (per_rank == nullptr) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "no rank descriptors given");
+  if (per_rank[0].cp_size != cp_size || per_rank[0].cp_rank != 0)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "loopback needs descriptors of ranks 0..cp_size-1 in order");
+  Plan plan;
+  int rc = build_plan(per_rank, cp_size, true, &plan);
+  if (rc) return rc;
+  return launch_rounds(plan, true, true, true, static_cast<hipStream_t>(stream));
+}
+
+int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t*, const helix_a2a_combine_out_t*, int, int, int,
+                                        void*) {
+  return fail(HELIX_A2A_ERR_RUNTIME, "fused combine is not built into this library");
+}
+
+int helix_a2a_device_status(uint32_t* status, void* stream) {
+  if (status == nullptr) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "status pointer is null");
+  DeviceState* st = nullptr;
+  int rc = device_state(&st);
+  if (rc) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  HELIX_HIP_TRY(hipStreamSynchronize(s));
+  uint32_t host = 0;
+  HELIX_HIP_TRY(hipMemcpy(&host, st->status, sizeof(host), hipMemcpyDeviceToHost));
+  if (host != 0) HELIX_HIP_TRY(hipMemset(st->status, 0, sizeof(uint32_t)));
+  *status = host;
+  return HELIX_A2A_OK;
+}
+
+void helix_a2a_set_spin_limit_us(uint64_t microseconds) { g_spinLimitUs.store(microseconds); }
+
+void helix_a2a_set_single_round(int enabled) { g_singleRound.store(enabled ? 1 : 0); }
+
+const char* helix_a2a_last_error(void) { return g_lastError; }
+
+const char* helix_a2a_version(void) { return "0.1.0"; }
+
+}  // extern "C"

@@ -1,0 +1,52 @@
+// helix_kernels.hpp -- launch descriptors shared by the kernels and the host
+// side of the library (internal; the public boundary is include/helix_a2a.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "helix_ll128.hpp"
+
+namespace helix {
+
+// Field pointers of one logical rank.
+struct RankPtrs {
+  const uint8_t* send0;  // partial_o     [E, cp, field0Bytes]
+  const uint8_t* send1;  // softmax_stats [E, cp, field1Bytes]
+  uint8_t* recv0;        // exchange: partial_o out; combine: combined out [E, field0Bytes]
+  uint8_t* recv1;        // exchange: softmax_stats out; combine: lse out [E, heads] or null
+};
+
+// Kernel argument block. `rank` is indexed by logical rank id; only ids in
+// [rankBegin, rankBegin + rankCount) are dereferenced by a launch.
+struct KernelArgs {
+  RankPtrs rank[kMaxCpSize];
+  uint8_t* workspace;       // base of the [cp, rowStrideBytes] workspace
+  uint64_t rowStrideBytes;
+  int cpSize;
+  int maxChannels;          // layout constant of the workspace
+  int runChannels;          // channels this launch deals entries over
+  int entryBegin, entryEnd; // entries [entryBegin, entryEnd) of the call
+  int field0Bytes, field1Bytes;
+  int sendStride0, sendStride1;  // bytes between consecutive (entry, peer) rows
+  int recvStride0, recvStride1;
+  int rankBegin, rankCount;
+  int doSend, doRecv;
+  uint64_t spinLimitTicks;  // bound of one in-kernel wait, in 100 MHz ticks
+  uint32_t* status;         // device status word (HELIX_A2A_STATUS_* bits)
+  // combine only
+  int heads, headDim;
+  int statsMode, dtype;
+};
+
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlockThreads = kWavesPerBlock * kWaveLanes;
+
+// wavefronts one direction of a launch needs: one per (local rank, channel, peer)
+inline int waves_per_direction(const KernelArgs& a) { return a.rankCount * a.runChannels * a.cpSize; }
+
+hipError_t launch_exchange(const KernelArgs& a, hipStream_t stream);
+hipError_t launch_combine_recv(const KernelArgs& a, hipStream_t stream);
+hipError_t launch_init_row(uint8_t* row, uint64_t fifoBytes, uint64_t infoBytes, hipStream_t stream);
+
+}  // namespace helix

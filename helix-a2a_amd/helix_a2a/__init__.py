@@ -1,0 +1,107 @@
+"""helix_a2a for MI355X: the Helix all-to-all behind the reference's Python API.
+
+The four public functions keep the names, argument order and error behaviour
+of the reference package (``helix_a2a/__init__.py:33-121``):
+
+    workspace_size(cp_size)                                   -> int (bytes per rank)
+    allocate_workspace(cp_size, cp_rank, device, *, mnnvl, cpu_group) -> int64 tensor [cp_size, elems]
+    init_workspace(workspace, cp_rank, cp_size)               -> None (synchronous)
+    alltoall(partial_o, softmax_stats, workspace, cp_rank, cp_size) -> (tensor, tensor)
+
+On one GPU the ``cp_size`` context-parallel ranks are logical ranks: row ``r``
+of the workspace tensor is rank ``r``'s FIFO memory, and all rows live in the
+same HBM. ``alltoall`` is called once per logical rank; the outputs of every
+rank are complete once all ``cp_size`` ranks have made their call and the
+stream has drained -- the single-device form of "every rank takes part".
+``alltoall_loopback`` issues all ranks in one fused launch.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+from helix_a2a import _ops
+from helix_a2a._ops import STATS_LSE, STATS_MAX_SUM  # noqa: F401
+from helix_a2a._version import __version__  # noqa: F401
+
+__all__ = [
+    "workspace_size",
+    "allocate_workspace",
+    "init_workspace",
+    "alltoall",
+    "alltoall_loopback",
+]
+
+
+def workspace_size(cp_size: int) -> int:
+    """Bytes of workspace one rank needs on the current device.
+
+    ``(512 KiB + 2 * 256 B) * cp_size * max_channels`` with
+    ``max_channels = max(CUs // (2 * ceil(cp_size / 8)), 1)``
+    (the reference's formula with the CU count as its SM count,
+    ``csrc/helix_alltoall.cu:590-614``).
+    """
+    return _ops.get_workspace_size_per_rank(cp_size)
+
+
+def allocate_workspace(
+    cp_size: int,
+    cp_rank: int,
+    device: str = "cuda",
+    *,
+    mnnvl: "bool | str" = False,
+    cpu_group=None,
+) -> torch.Tensor:
+    """Allocate the ``[cp_size, elems_per_rank]`` int64 workspace in device memory.
+
+    Follow it with :func:`init_workspace` for every logical rank before the
+    first exchange. ``mnnvl`` selects the reference's NVIDIA fabric-handle
+    allocator (``helix_a2a/mnnvl.py``), which has no single-GPU counterpart:
+    ``True`` raises, ``"auto"`` resolves to plain device memory.
+    """
+    if mnnvl is True:
+        raise RuntimeError("MNNVL workspaces need NVIDIA fabric handles; this build places all "
+                           "logical ranks in one device allocation (pass mnnvl=False)")
+    del cp_rank, cpu_group  # every row lives in the same allocation
+    elems = (workspace_size(cp_size) + 7) // 8
+    return torch.zeros(cp_size, elems, dtype=torch.int64, device=device)
+
+
+def init_workspace(workspace: torch.Tensor, cp_rank: int, cp_size: int) -> None:
+    """Reset the FIFOs and counters of row ``cp_rank``; returns once the GPU has done it.
+
+    All logical ranks must be initialised before any of them calls :func:`alltoall`.
+    Calling it again between exchanges is allowed (never while one is in flight).
+    """
+    _ops.initialize_workspace(workspace, cp_rank, cp_size)
+    torch.cuda.current_stream().synchronize()
+
+
+def alltoall(
+    partial_o: torch.Tensor,
+    softmax_stats: torch.Tensor,
+    workspace: torch.Tensor,
+    cp_rank: int,
+    cp_size: int,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Helix all-to-all of one rank.
+
+    ``partial_o`` is ``[..., cp_size, D]`` (fp16/bf16), ``softmax_stats`` is
+    ``[..., cp_size, S]`` (fp32, S even); slice ``[..., p, :]`` goes to rank
+    ``p``. Returns tensors of the same shapes whose slice ``[..., p, :]`` came
+    from rank ``p``: ``out_r[e, s, :] = in_s[e, r, :]``, bit for bit.
+    Asynchronous on the current stream.
+    """
+    return _ops.alltoall_native(partial_o, softmax_stats, workspace, cp_rank, cp_size)
+
+
+def alltoall_loopback(
+    partial_o: Sequence[torch.Tensor],
+    softmax_stats: Sequence[torch.Tensor],
+    workspace: torch.Tensor,
+    channel_count: int = 0,
+    out: Optional[Tuple[Sequence[torch.Tensor], Sequence[torch.Tensor]]] = None,
+) -> Tuple[List[torch.Tensor], List[torch.Tensor]]:
+    """Exchange of all logical ranks in one launch: element ``r`` of each list is rank ``r``."""
+    return _ops.alltoall_loopback(partial_o, softmax_stats, workspace, channel_count, out)

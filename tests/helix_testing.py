@@ -1,0 +1,134 @@
+"""Helpers shared by the test modules (bit views, host-model front end, input builders)."""
+from __future__ import annotations
+
+import ctypes
+import subprocess
+from pathlib import Path
+from typing import List, Sequence, Tuple
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent.parent
+HOST_MODEL_DIR = ROOT / "tests" / "host_model"
+HOST_MODEL_LIB = HOST_MODEL_DIR / "libhelix_host_model.so"
+
+FIFO_BYTES = 512 * 1024
+FIFO_ENTRY_BYTES = 128 * 1024
+INFO_BYTES = 256
+
+
+def build_host_model() -> Path:
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-o", str(HOST_MODEL_LIB),
+           str(HOST_MODEL_DIR / "helix_host_model.cpp")]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("building the host model failed:\n" + proc.stdout + proc.stderr)
+    return HOST_MODEL_LIB
+
+
+class _Field(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("element_count", ctypes.c_int32),
+                ("element_size", ctypes.c_int32), ("stride_bytes", ctypes.c_int32)]
+
+
+class _Params(ctypes.Structure):
+    _fields_ = [("send_fields", _Field * 2), ("recv_fields", _Field * 2), ("entry_count", ctypes.c_int32),
+                ("workspace", ctypes.c_void_p), ("workspace_stride_u64", ctypes.c_uint64),
+                ("cp_rank", ctypes.c_int32), ("cp_size", ctypes.c_int32),
+                ("channel_count", ctypes.c_int32), ("max_channel_count", ctypes.c_int32)]
+
+
+class HostModel:
+    """ctypes front end of tests/host_model (the bounds-checked CPU walk-through of the GPU wave programs)."""
+
+    def __init__(self) -> None:
+        if not HOST_MODEL_LIB.exists():
+            build_host_model()
+        lib = ctypes.CDLL(str(HOST_MODEL_LIB))
+        lib.hm_alltoall.argtypes = [ctypes.POINTER(_Params)] + [ctypes.c_int] * 5
+        lib.hm_alltoall.restype = ctypes.c_int
+        lib.hm_last_message.restype = ctypes.c_char_p
+        for name in ("hm_fifo_offset",):
+            getattr(lib, name).argtypes = [ctypes.c_int] * 3
+            getattr(lib, name).restype = ctypes.c_uint64
+        for name in ("hm_sender_info_offset", "hm_receiver_info_offset"):
+            getattr(lib, name).argtypes = [ctypes.c_int] * 4
+            getattr(lib, name).restype = ctypes.c_uint64
+        lib.hm_msg_lines.argtypes = [ctypes.c_int, ctypes.c_int]
+        lib.hm_msg_lines.restype = ctypes.c_int
+        lib.hm_unit_first_piece.argtypes = [ctypes.c_int]
+        lib.hm_unit_first_piece.restype = ctypes.c_int
+        self.lib = lib
+
+    @staticmethod
+    def max_channel_count(cp: int, cu_count: int) -> int:
+        return max(cu_count // (2 * -(-cp // 8)), 1)
+
+    def new_workspace(self, cp: int, cu_count: int, init: bool = True) -> np.ndarray:
+        ch = self.max_channel_count(cp, cu_count)
+        fifo_elems = FIFO_BYTES * cp * ch // 8
+        info_elems = 2 * INFO_BYTES * cp * ch // 8
+        ws = np.zeros((cp, fifo_elems + info_elems), dtype=np.int64)
+        if init:
+            ws[:, :fifo_elems] = -1
+        return ws
+
+    def alltoall(self, ins_o: Sequence[np.ndarray], ins_s: Sequence[np.ndarray], workspace: np.ndarray,
+                 cu_count: int, channels: int, send: bool = True, recv: bool = True,
+                 outs: Tuple[List[np.ndarray], List[np.ndarray]] | None = None,
+                 ) -> Tuple[List[np.ndarray], List[np.ndarray], int, str]:
+        cp = len(ins_o)
+        if outs is None:
+            outs = ([np.zeros_like(a) for a in ins_o], [np.zeros_like(a) for a in ins_s])
+        arr = (_Params * cp)()
+        for r in range(cp):
+            p = arr[r]
+            for f, (src, dst) in enumerate(((ins_o[r], outs[0][r]), (ins_s[r], outs[1][r]))):
+                for field, a in ((p.send_fields[f], src), (p.recv_fields[f], dst)):
+                    assert a.ndim == 3 and a.flags["C_CONTIGUOUS"]
+                    field.data = a.ctypes.data
+                    field.element_count = a.shape[2]
+                    field.element_size = a.itemsize
+                    field.stride_bytes = a.strides[1]
+            p.entry_count = ins_o[r].shape[0]
+            p.workspace = workspace.ctypes.data
+            p.workspace_stride_u64 = workspace.strides[0] // 8
+            p.cp_rank, p.cp_size = r, cp
+            p.channel_count = channels
+            p.max_channel_count = self.max_channel_count(cp, cu_count)
+        rc = self.lib.hm_alltoall(arr, cp, cu_count, channels, int(send), int(recv))
+        return outs[0], outs[1], rc, self.lib.hm_last_message().decode()
+
+
+# ---------------------------------------------------------------------------
+# bit views
+# ---------------------------------------------------------------------------
+
+def torch_bits(t) -> np.ndarray:
+    """Raw bit pattern of a torch tensor as an unsigned numpy array (bf16/fp16 -> uint16, fp32 -> uint32)."""
+    import torch
+
+    t = t.detach().cpu().contiguous()
+    view = {2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()]
+    unsigned = {2: np.uint16, 4: np.uint32, 8: np.uint64}[t.element_size()]
+    return t.view(view).numpy().view(unsigned)
+
+
+def coded_inputs(cp: int, entries: int, x: int, s: int) -> Tuple[List[np.ndarray], List[np.ndarray]]:
+    """Integer-coded payloads: every 2-byte / 4-byte element names its (rank, entry, peer, index)."""
+    ins_o, ins_s = [], []
+    for r in range(cp):
+        e, p, i = np.meshgrid(np.arange(entries), np.arange(cp), np.arange(x), indexing="ij")
+        o = (r * 4099 + e * 523 + p * 67 + i) & 0xFFFF
+        ins_o.append(o.astype(np.uint16))
+        e, p, i = np.meshgrid(np.arange(entries), np.arange(cp), np.arange(s), indexing="ij")
+        st = (r << 24) | (e << 12) | (p << 8) | i
+        ins_s.append(st.astype(np.uint32))
+    return ins_o, ins_s
+
+
+def random_inputs(cp: int, entries: int, x: int, s: int, seed: int) -> Tuple[List[np.ndarray], List[np.ndarray]]:
+    rng = np.random.default_rng(seed)
+    ins_o = [rng.integers(0, 1 << 16, size=(entries, cp, x), dtype=np.uint16) for _ in range(cp)]
+    ins_s = [rng.integers(0, 1 << 32, size=(entries, cp, s), dtype=np.uint32) for _ in range(cp)]
+    return ins_o, ins_s

@@ -1,0 +1,234 @@
+// helix_host_model.cpp -- CPU walk-through of the GPU kernels' wave programs.
+//
+// Test fixture (never loaded by the product). It executes, lane by lane and
+// in plain C++, the same sequence of loads and stores the gfx950 kernels
+// issue, using the index arithmetic of csrc/helix_ll128.hpp, on host memory,
+// and checks every single access against the extent of the buffer it
+// belongs to. CPU tests use it to show that the index math stays in bounds
+// for a shape before that shape is ever launched on a GPU, and to produce the
+// expected FIFO image (line layout, flags, counters) that GPU tests compare
+// the real FIFO contents with.
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/helix_a2a.h"
+#include "../../helix-a2a_amd/csrc/helix_ll128.hpp"
+
+using namespace helix;
+
+namespace {
+
+struct Extent {
+  const uint8_t* base;
+  uint64_t bytes;
+};
+
+struct Checker {
+  int violations = 0;
+  int outOfExtent = 0;
+  char first[256] = "";
+  bool ok(const Extent& e, const void* p, uint64_t n, const char* what) {
+    const uint8_t* q = static_cast<const uint8_t*>(p);
+    if (q >= e.base && q + n <= e.base + e.bytes) return true;
+    outOfExtent++;
+    if (violations++ == 0)
+      snprintf(first, sizeof(first), "%s: access of %llu bytes at offset %lld outside extent %llu", what,
+               (unsigned long long)n, (long long)(q - e.base), (unsigned long long)e.bytes);
+    return false;
+  }
+};
+
+thread_local char g_msg[256] = "";
+thread_local int g_outOfExtent = 0;
+
+struct Ctx {
+  const helix_a2a_params_t* ranks;
+  int cp, maxCh, channels, entryBegin, entryEnd;
+  MsgShape sh;
+  Extent ws;
+  Checker chk;
+};
+
+Extent field_extent(const helix_a2a_field_t& f, int entries, int cp) {
+  return Extent{static_cast<const uint8_t*>(f.data), static_cast<uint64_t>(entries) * cp * f.stride_bytes};
+}
+
+// sender wave of stream (s -> r, ch)
+void run_sender(Ctx& c, int s, int r, int ch) {
+  const helix_a2a_params_t& p = c.ranks[s];
+  uint8_t* wsBase = reinterpret_cast<uint8_t*>(p.workspace);
+  uint64_t rowStride = p.workspace_stride_u64 * 8;
+  uint8_t* senderRow = wsBase + s * rowStride;
+  uint8_t* receiverRow = wsBase + r * rowStride;
+  int64_t* info = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(c.cp, c.maxCh, r, ch));
+  uint8_t* fifo = receiverRow + fifo_offset(s, ch, c.maxCh);
+  if (!c.chk.ok(c.ws, info, 16, "sender info") || !c.chk.ok(c.ws, fifo, kFifoBytes, "fifo")) return;
+  Extent fifoExt{fifo, kFifoBytes};
+  Extent e0 = field_extent(p.send_fields[0], p.entry_count, c.cp);
+  Extent e1 = field_extent(p.send_fields[1], p.entry_count, c.cp);
+  FifoCursor cur = make_cursor(info[0]);
+  for (int e = c.entryBegin + ch; e < c.entryEnd; e += c.channels) {
+    if (cursor_needs_new_entry(cur, c.sh.lines)) {
+      bool closed;
+      cursor_open_entry(cur, &closed);
+      if (closed) info[0] = cur.step;
+      // the model runs senders to completion first: room must already be there
+      if (info[1] + kFifoDepth <= cur.step) {
+        c.chk.violations++;
+        snprintf(c.chk.first, sizeof(c.chk.first), "sender %d->%d ch %d would block at step %lld", s, r, ch,
+                 (long long)cur.step);
+        return;
+      }
+    }
+    uint64_t row = static_cast<uint64_t>(e) * c.cp + r;
+    const uint8_t* row0 = e0.base + row * p.send_fields[0].stride_bytes;
+    const uint8_t* row1 = e1.base + row * p.send_fields[1].stride_bytes;
+    uint32_t msgOff = fifo_unit_offset(cursor_entry_index(cur), cur.lineBase, 0);
+    for (int g = 0; g < c.sh.units; ++g) {  // every lane of every wave access
+      uint64_t words[2] = {0, 0};
+      int p0 = unit_first_piece(g);
+      for (int k = 0; k < 2; ++k) {
+        int piece = p0 + k;
+        if (k == 1 && unit_has_flag(g)) {
+          words[1] = static_cast<uint64_t>(cur.step);
+        } else if (piece < c.sh.np0) {
+          const uint8_t* src = row0 + piece * kPieceBytes;
+          if (c.chk.ok(e0, src, 8, "send field 0")) memcpy(&words[k], src, 8);
+        } else if (piece < c.sh.np) {
+          const uint8_t* src = row1 + (piece - c.sh.np0) * kPieceBytes;
+          if (c.chk.ok(e1, src, 8, "send field 1")) memcpy(&words[k], src, 8);
+        }
+      }
+      uint8_t* dst = fifo + msgOff + g * kUnitBytes;
+      if (c.chk.ok(fifoExt, dst, 16, "fifo store")) memcpy(dst, words, 16);
+    }
+    cur.lineBase += c.sh.lines;
+  }
+  if (cur.open) info[0] = cur.step + 1;
+}
+
+// receiver wave of stream (s -> r, ch); a line whose flag is not there counts as a violation
+void run_receiver(Ctx& c, int r, int s, int ch) {
+  const helix_a2a_params_t& p = c.ranks[r];
+  uint8_t* wsBase = reinterpret_cast<uint8_t*>(p.workspace);
+  uint64_t rowStride = p.workspace_stride_u64 * 8;
+  uint8_t* senderRow = wsBase + s * rowStride;
+  uint8_t* receiverRow = wsBase + r * rowStride;
+  int64_t* sinfo = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(c.cp, c.maxCh, r, ch));
+  int64_t* info = reinterpret_cast<int64_t*>(receiverRow + receiver_info_offset(c.cp, c.maxCh, s, ch));
+  uint8_t* fifo = receiverRow + fifo_offset(s, ch, c.maxCh);
+  if (!c.chk.ok(c.ws, info, 16, "receiver info") || !c.chk.ok(c.ws, sinfo, 16, "sender info") ||
+      !c.chk.ok(c.ws, fifo, kFifoBytes, "fifo"))
+    return;
+  Extent fifoExt{fifo, kFifoBytes};
+  Extent e0 = field_extent(p.recv_fields[0], p.entry_count, c.cp);
+  Extent e1 = field_extent(p.recv_fields[1], p.entry_count, c.cp);
+  FifoCursor cur = make_cursor(info[1]);
+  for (int e = c.entryBegin + ch; e < c.entryEnd; e += c.channels) {
+    if (cursor_needs_new_entry(cur, c.sh.lines)) {
+      bool closed;
+      cursor_open_entry(cur, &closed);
+      if (closed) {
+        info[1] = cur.step;
+        sinfo[1] = cur.step;
+      }
+    }
+    uint64_t row = static_cast<uint64_t>(e) * c.cp + s;
+    uint8_t* row0 = const_cast<uint8_t*>(e0.base) + row * p.recv_fields[0].stride_bytes;
+    uint8_t* row1 = const_cast<uint8_t*>(e1.base) + row * p.recv_fields[1].stride_bytes;
+    uint32_t msgOff = fifo_unit_offset(cursor_entry_index(cur), cur.lineBase, 0);
+    for (int g = 0; g < c.sh.units; ++g) {
+      const uint8_t* src = fifo + msgOff + g * kUnitBytes;
+      if (!c.chk.ok(fifoExt, src, 16, "fifo load")) continue;
+      uint64_t words[2];
+      memcpy(words, src, 16);
+      // flag of this lane's line
+      uint64_t flag;
+      memcpy(&flag, fifo + msgOff + (g | 7) * kUnitBytes + 8, 8);
+      if (flag != static_cast<uint64_t>(cur.step)) {
+        if (c.chk.violations++ == 0)
+          snprintf(c.chk.first, sizeof(c.chk.first), "stream %d->%d ch %d entry %d: flag %llx != step %llx", s, r, ch,
+                   e, (unsigned long long)flag, (unsigned long long)cur.step);
+        continue;
+      }
+      int p0 = unit_first_piece(g);
+      for (int k = 0; k < 2; ++k) {
+        int piece = p0 + k;
+        if (k == 1 && unit_has_flag(g)) break;
+        if (piece < c.sh.np0) {
+          uint8_t* dst = row0 + piece * kPieceBytes;
+          if (c.chk.ok(e0, dst, 8, "recv field 0")) memcpy(dst, &words[k], 8);
+        } else if (piece < c.sh.np) {
+          uint8_t* dst = row1 + (piece - c.sh.np0) * kPieceBytes;
+          if (c.chk.ok(e1, dst, 8, "recv field 1")) memcpy(dst, &words[k], 8);
+        }
+      }
+    }
+    cur.lineBase += c.sh.lines;
+  }
+  if (cur.open) {
+    info[1] = cur.step + 1;
+    sinfo[1] = cur.step + 1;
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* hm_last_message(void) { return g_msg; }
+// accesses the last hm_alltoall refused because they left their buffer
+int hm_last_out_of_extent(void) { return g_outOfExtent; }
+
+// Run the send and/or receive programs of all cp ranks (per_rank[r].cp_rank == r)
+// for entries [0, entry_count) split in rounds exactly like the library does.
+// Returns the number of violations (out-of-extent accesses, missing flags,
+// blocked senders); 0 means the walk-through was clean.
+int hm_alltoall(const helix_a2a_params_t* per_rank, int cp, int cu_count, int channels, int do_send, int do_recv) {
+  g_msg[0] = 0;
+  Ctx c;
+  c.ranks = per_rank;
+  c.cp = cp;
+  c.maxCh = max_channel_count(cp, cu_count);
+  c.channels = channels;
+  const helix_a2a_params_t& p0 = per_rank[0];
+  c.sh = make_msg_shape(p0.send_fields[0].element_count * p0.send_fields[0].element_size,
+                        p0.send_fields[1].element_count * p0.send_fields[1].element_size);
+  c.ws = Extent{reinterpret_cast<const uint8_t*>(p0.workspace), p0.workspace_stride_u64 * 8 * cp};
+  if (channels < 1 || channels > c.maxCh || c.sh.lines > kFifoEntryLines) {
+    snprintf(g_msg, sizeof(g_msg), "bad channel count or message size");
+    return -1;
+  }
+  long perStream = static_cast<long>(kFifoDepth) * msgs_per_fifo_entry(c.sh);
+  long roundEntries = perStream * channels;
+  for (long begin = 0; begin < p0.entry_count; begin += roundEntries) {
+    c.entryBegin = static_cast<int>(begin);
+    long end = begin + roundEntries;
+    c.entryEnd = end > p0.entry_count ? p0.entry_count : static_cast<int>(end);
+    if (do_send)
+      for (int s = 0; s < cp; ++s)
+        for (int ch = 0; ch < channels; ++ch)
+          for (int r = 0; r < cp; ++r) run_sender(c, s, r, ch);
+    if (do_recv)
+      for (int r = 0; r < cp; ++r)
+        for (int ch = 0; ch < channels; ++ch)
+          for (int s = 0; s < cp; ++s) run_receiver(c, r, s, ch);
+  }
+  if (c.chk.violations) snprintf(g_msg, sizeof(g_msg), "%s", c.chk.first);
+  g_outOfExtent = c.chk.outOfExtent;
+  return c.chk.violations;
+}
+
+// geometry probes for tests
+uint64_t hm_fifo_offset(int sender, int channel, int max_ch) { return fifo_offset(sender, channel, max_ch); }
+uint64_t hm_sender_info_offset(int cp, int max_ch, int receiver, int channel) {
+  return sender_info_offset(cp, max_ch, receiver, channel);
+}
+uint64_t hm_receiver_info_offset(int cp, int max_ch, int sender, int channel) {
+  return receiver_info_offset(cp, max_ch, sender, channel);
+}
+int hm_msg_lines(int f0, int f1) { return make_msg_shape(f0, f1).lines; }
+int hm_unit_first_piece(int g) { return unit_first_piece(g); }
+
+}  // extern "C"

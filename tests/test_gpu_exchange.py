@@ -1,0 +1,505 @@
+"""GPU parity tests of the exchange: the HIP path, called through the C ABI, against the oracle.
+
+Bit-exact everywhere: the exchange moves opaque bytes.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helix_testing import FIFO_BYTES, torch_bits
+from oracle import helix_oracle as ho
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hx():
+    import helix_a2a
+
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return helix_a2a
+
+
+@pytest.fixture(scope="module")
+def ops(hx):
+    from helix_a2a import _ops
+
+    return _ops
+
+
+_WORKSPACES = {}
+
+
+def get_workspace(hx, cp, fresh=False):
+    """One workspace per cp for the whole module (4.3 GB at cp = 8), initialised on first use."""
+    ws = _WORKSPACES.get(cp)
+    if ws is None:
+        ws = _WORKSPACES[cp] = hx.allocate_workspace(cp, 0)
+        fresh = True
+    if fresh:
+        for r in range(cp):
+            hx.init_workspace(ws, r, cp)
+    return ws
+
+
+def bits_equal(a: torch.Tensor, b: torch.Tensor) -> bool:
+    view = {2: torch.int16, 4: torch.int32}[a.element_size()]
+    return torch.equal(a.contiguous().view(view), b.contiguous().view(view))
+
+
+def expected_on_device(ins):
+    """The oracle's single-copy form of the closed form, evaluated on the tensors' device."""
+    return ho.exchange_single_copy(ins)
+
+
+def check_against_oracle(ins_o, ins_s, outs_o, outs_s, with_numpy=True):
+    cp = len(ins_o)
+    want_o, want_s = expected_on_device(ins_o), expected_on_device(ins_s)
+    for r in range(cp):
+        assert bits_equal(outs_o[r].view(ins_o[r].shape), want_o[r]), f"partial_o of rank {r} differs"
+        assert bits_equal(outs_s[r].view(ins_s[r].shape), want_s[r]), f"softmax_stats of rank {r} differs"
+    if with_numpy:  # the same comparison on the host against the numpy closed form, on raw bits
+        np_o = ho.exchange_closed_form([torch_bits(t) for t in ins_o])
+        np_s = ho.exchange_closed_form([torch_bits(t) for t in ins_s])
+        for r in range(cp):
+            assert np.array_equal(torch_bits(outs_o[r]).reshape(np_o[r].shape), np_o[r])
+            assert np.array_equal(torch_bits(outs_s[r]).reshape(np_s[r].shape), np_s[r])
+
+
+def assert_clean(ops):
+    assert ops.device_status() == 0, "a kernel reported a timed-out wait"
+
+
+# ---------------------------------------------------------------------------
+# the reference's single-GPU tests (tests/test_build.py, tests/test_phase2.py)
+# ---------------------------------------------------------------------------
+
+def _max_channels(cp_size):
+    cu = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+    max_group = min(cp_size, 8)
+    blocks_per_ch = ((cp_size + max_group - 1) // max_group) * 2
+    return max(cu // blocks_per_ch, 1)
+
+
+def test_workspace_size_matches_manual_computation(hx):
+    for cp_size in (2, 4, 8):
+        ch = _max_channels(cp_size)
+        expected = 512 * 1024 * cp_size * ch + 256 * cp_size * ch * 2
+        actual = hx.workspace_size(cp_size)
+        assert isinstance(actual, int) and actual == expected
+    assert hx.workspace_size(4) != 16_778_240
+
+
+def test_init_workspace_pattern(hx):
+    cp = 4
+    ws = hx.allocate_workspace(cp_size=cp, cp_rank=0)
+    assert ws.dtype == torch.int64 and ws.dim() == 2 and ws.shape[0] == cp and ws.shape[1] > 0
+    ws.fill_(0x1234)
+    hx.init_workspace(ws, cp_rank=2, cp_size=cp)
+    fifo_elems = 512 * 1024 * cp * _max_channels(cp) // 8
+    assert bool((ws[2, :fifo_elems] == -1).all())
+    assert bool((ws[2, fifo_elems:] == 0).all())
+    for other in (0, 1, 3):
+        assert bool((ws[other] == 0x1234).all())
+    del ws
+    torch.cuda.empty_cache()
+
+
+def test_input_validation(hx):
+    cp = 4
+    ws = get_workspace(hx, cp)
+    good_o = torch.randn(2, cp, 128, dtype=torch.bfloat16, device="cuda")
+    good_s = torch.randn(2, cp, 2, dtype=torch.float32, device="cuda")
+    bad = [
+        (good_o.float(), good_s, ws, 0, cp),                                        # partial_o dtype
+        (good_o, good_s.half(), ws, 0, cp),                                         # stats dtype
+        (torch.randn(2, 3, 128, dtype=torch.bfloat16, device="cuda"), good_s, ws, 0, cp),  # cp dimension
+        (good_o, torch.randn(2, cp, 3, device="cuda"), ws, 0, cp),                  # odd stats width
+        (good_o, torch.randn(3, cp, 2, device="cuda"), ws, 0, cp),                  # leading dims differ
+        (torch.randn(2, cp, 100, dtype=torch.bfloat16, device="cuda"), good_s, ws, 0, cp),  # 200-byte rows
+        (good_o.transpose(0, 1), good_s, ws, 0, cp),                                # not contiguous
+        (good_o, good_s, ws.int(), 0, cp),                                          # workspace dtype
+        (good_o, good_s, ws[0], 0, cp),                                             # workspace rank
+        (good_o, good_s, ws[:2], 0, cp),                                            # workspace rows
+        (good_o, good_s, ws, cp, cp),                                               # rank out of range
+        (good_o, good_s, ws, -1, cp),
+        (good_o.cpu(), good_s, ws, 0, cp),
+    ]
+    for args in bad:
+        with pytest.raises(RuntimeError):
+            hx.alltoall(*args)
+    with pytest.raises(RuntimeError):
+        hx.init_workspace(ws, cp, cp)
+    with pytest.raises(RuntimeError):
+        hx.init_workspace(ws[:, :1000], 0, cp)
+    # nothing was enqueued by the rejected calls
+    from helix_a2a import _ops
+    assert not any(g.pending for g in _ops._groups.values())
+
+
+# ---------------------------------------------------------------------------
+# loopback parity on the benchmark workloads
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c5b", "c3", "c4", "c5a"])
+def test_loopback_workloads(hx, ops, name):
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS[name]
+    ws = get_workspace(hx, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws)
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(ins_o, ins_s, outs_o, outs_s, with_numpy=name in ("c1", "c2", "c5b", "c3"))
+
+
+@pytest.mark.parametrize("name", ["c1", "c5b", "c2"])
+def test_loopback_against_reference_model(hx, ops, ref_model, name):
+    # the C restatement of the reference kernel, run on the same bits
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS[name]
+    ws = get_workspace(hx, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws)
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    np_o, np_s = [torch_bits(t) for t in ins_o], [torch_bits(t) for t in ins_s]
+    model_ws = ref_model.new_workspace(w.cp, 8)
+    for r in range(w.cp):
+        ref_model.init_workspace(model_ws, r, w.cp, 8)
+    ref_o, ref_s = ref_model.alltoall_all_ranks(np_o, np_s, model_ws, sm_count=8)
+    for r in range(w.cp):
+        assert np.array_equal(torch_bits(outs_o[r]), ref_o[r])
+        assert np.array_equal(torch_bits(outs_s[r]), ref_s[r])
+
+
+@pytest.mark.parametrize("name", ["c2", "c5b", "c3"])
+def test_per_head_layout(hx, ops, name):
+    # the layout the serving integration passes: one entry per (token, head), stats are one float2
+    from helix_a2a.workloads import WORKLOADS, as_head_layout, make_inputs
+
+    w = WORKLOADS[name]
+    ws = get_workspace(hx, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    pairs = [as_head_layout(w, o, s) for o, s in zip(ins_o, ins_s)]
+    h_o, h_s = [p[0] for p in pairs], [p[1] for p in pairs]
+    assert h_s[0].shape[-1] == 2
+    outs_o, outs_s = hx.alltoall_loopback(h_o, h_s, ws)
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(h_o, h_s, outs_o, outs_s, with_numpy=name != "c3")
+
+
+@pytest.mark.parametrize("channels", [1, 2, 3, 4, 8, 16, 32, 64, 128, 0])
+def test_channel_sweep(hx, ops, channels):
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS["c3"]
+    ws = get_workspace(hx, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws, channel_count=channels)
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(ins_o, ins_s, outs_o, outs_s, with_numpy=False)
+
+
+def test_channel_count_limits(hx, ops):
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS["c1"]
+    ws = get_workspace(hx, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    with pytest.raises(RuntimeError, match="channel_count"):
+        hx.alltoall_loopback(ins_o, ins_s, ws, channel_count=ops.max_channel_count(w.cp) + 1)
+    os.environ["HELIX_A2A_CHANNEL_COUNT"] = "3"
+    try:
+        outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws)
+        torch.cuda.synchronize()
+    finally:
+        del os.environ["HELIX_A2A_CHANNEL_COUNT"]
+    assert_clean(ops)
+    check_against_oracle(ins_o, ins_s, outs_o, outs_s)
+
+
+@pytest.mark.parametrize("cp,entries,x,s", [
+    (4, 37, 48, 2),     # 104 bytes: a single partial line
+    (3, 11, 8, 6),      # 40 bytes, odd cp, stats row of 24 bytes
+    (2, 1, 8, 2),       # smallest legal message: 24 bytes
+    (5, 13, 136, 10),   # 312 bytes: 2.6 lines, straddling units
+    (7, 3, 2048, 62),   # 4344 bytes
+    (2, 4, 61440, 2),   # 122888 bytes: 1025 lines, more than a FIFO entry holds -> rejected
+    (1, 9, 64, 2),      # a single rank talking to itself
+    (16, 2, 64, 2),
+    (4, 0, 64, 2),      # nothing to send
+])
+def test_ragged_shapes(hx, ops, cp, entries, x, s):
+    ws = get_workspace(hx, cp)
+    g = torch.Generator().manual_seed(cp * 1000 + entries)
+    ins_o = [torch.randint(-32768, 32767, (entries, cp, x), generator=g, dtype=torch.int16).view(torch.bfloat16).cuda()
+             for _ in range(cp)]
+    ins_s = [torch.randint(-2**31, 2**31 - 1, (entries, cp, s), generator=g, dtype=torch.int32).view(torch.float32).cuda()
+             for _ in range(cp)]
+    if 2 * x + 4 * s > 1024 * 120:
+        with pytest.raises(RuntimeError, match="FIFO entry"):
+            hx.alltoall_loopback(ins_o, ins_s, ws)
+        return
+    outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws)
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    if entries:
+        check_against_oracle(ins_o, ins_s, outs_o, outs_s)
+    else:
+        assert outs_o[0].shape == ins_o[0].shape
+
+
+def test_special_values_survive(hx, ops):
+    # NaN payloads, infinities, denormals and negative zero are bytes like any other
+    cp, entries = 2, 4
+    ws = get_workspace(hx, cp)
+    specials = torch.tensor([float("nan"), float("inf"), float("-inf"), -0.0, 1e-45, 3.0e38, 0.0, -1.0])
+    ins_o = [specials.to(torch.bfloat16).repeat(entries, cp, 16).cuda() for _ in range(cp)]
+    ins_s = [specials.repeat(entries, cp, 1).contiguous().cuda() for _ in range(cp)]
+    ins_s[1] = ins_s[1].view(torch.int32).bitwise_xor(0x00400001).view(torch.float32)  # a signalling-NaN pattern among them
+    outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws)
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(ins_o, ins_s, outs_o, outs_s)
+
+
+# ---------------------------------------------------------------------------
+# FIFO state across calls
+# ---------------------------------------------------------------------------
+
+def test_repeated_calls_wrap_the_fifo(hx, ops):
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS["c2"]
+    ws = get_workspace(hx, w.cp, fresh=True)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    for call in range(11):  # every stream consumes one FIFO entry per call: entries are reused from call 4 on
+        rolled_o = [t.roll(call, 0) for t in ins_o]
+        rolled_s = [t.roll(call, 0) for t in ins_s]
+        outs_o, outs_s = hx.alltoall_loopback(rolled_o, rolled_s, ws, channel_count=(call % 5) * 7 + 1)
+        check_against_oracle(rolled_o, rolled_s, outs_o, outs_s, with_numpy=False)
+    assert_clean(ops)
+
+
+def test_reinit_between_calls(hx, ops):
+    # tests/test_mnnvl.py:100-161 re-initialises the workspace before every call
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS["c1"]
+    ws = get_workspace(hx, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    for _ in range(3):
+        for r in range(w.cp):
+            hx.init_workspace(ws, r, w.cp)
+        outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws)
+        check_against_oracle(ins_o, ins_s, outs_o, outs_s)
+    assert_clean(ops)
+
+
+def test_many_calls_back_to_back_without_sync(hx, ops):
+    # a torn or stale line would show up as a mismatch in one of many asynchronous iterations
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS["c3"]
+    ws = get_workspace(hx, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    want_o, want_s = expected_on_device(ins_o), expected_on_device(ins_s)
+    bad = torch.zeros((), dtype=torch.int64, device="cuda")
+    for it in range(60):
+        src_o = [t.bitwise_xor(it) for t in (x.view(torch.int16) for x in ins_o)]
+        outs_o, outs_s = hx.alltoall_loopback([t.view(torch.bfloat16) for t in src_o], ins_s, ws)
+        for r in range(w.cp):
+            bad += (outs_o[r].view(torch.int16) != want_o[r].view(torch.int16).bitwise_xor(it)).sum()
+            bad += (outs_s[r].view(torch.int32) != want_s[r].view(torch.int32)).sum()
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    assert int(bad.item()) == 0
+
+
+# ---------------------------------------------------------------------------
+# the per-rank call (the reference's signature)
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_per_rank_calls_seeded_full_tensor(hx, ops, dtype):
+    # tests/test_alltoall.py:303-360 on logical ranks: rank r sends full[:, :, r, :] and receives full[:, r, :, :]
+    cp, b, d, s = 4, 4, 128, 2
+    ws = get_workspace(hx, cp)
+    torch.manual_seed(42)
+    full_o = torch.randn(b, cp, cp, d, dtype=dtype, device="cuda")
+    full_s = torch.randn(b, cp, cp, s, dtype=torch.float32, device="cuda")
+    results = []
+    for rank in range(cp):
+        send_o = full_o[:, :, rank, :].contiguous()
+        send_s = full_s[:, :, rank, :].contiguous()
+        results.append(hx.alltoall(send_o.clone(), send_s.clone(), ws, cp_rank=rank, cp_size=cp))
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    for rank, (recv_o, recv_s) in enumerate(results):
+        assert bits_equal(recv_o, full_o[:, rank, :, :])
+        assert bits_equal(recv_s, full_s[:, rank, :, :])
+
+
+def test_per_rank_calls_fill_vectors(hx, ops):
+    # tests/test_mnnvl.py:164-219: rank r sends the constant r+1; slot j of every result holds j+1
+    cp, n, d = 4, 4, 64
+    ws = get_workspace(hx, cp)
+    results = []
+    for rank in reversed(range(cp)):  # any call order works
+        po = torch.full((n, cp, d), float(rank + 1), dtype=torch.bfloat16, device="cuda")
+        ss = torch.full((n, cp, 2), float(rank + 1) * 0.1, dtype=torch.float32, device="cuda")
+        results.append((rank, *hx.alltoall(po, ss, ws, cp_rank=rank, cp_size=cp)))
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    for rank, po_out, ss_out in results:
+        assert po_out.shape == (n, cp, d) and ss_out.shape == (n, cp, 2)
+        for j in range(cp):
+            assert bool((po_out[:, j, :].float() == float(j + 1)).all())
+            assert bool((ss_out[:, j, :] == torch.tensor(float(j + 1) * 0.1, dtype=torch.float32)).all())
+
+
+def test_per_rank_calls_4d_and_leading_dims(hx, ops):
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS["c2"]
+    ws = get_workspace(hx, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    hp = w.heads_per_rank
+    outs = [hx.alltoall(o.view(w.tokens, w.cp, hp, w.head_dim), s.view(w.tokens, w.cp, hp, 2), ws, r, w.cp)
+            for r, (o, s) in enumerate(zip(ins_o, ins_s))]
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    assert outs[0][0].shape == (w.tokens, w.cp, hp, w.head_dim)
+    check_against_oracle(ins_o, ins_s, [o[0] for o in outs], [o[1] for o in outs], with_numpy=False)
+    # extra leading dimensions are flattened into the entry count: [2, T/2, cp, X]
+    outs = [hx.alltoall(o.view(2, w.tokens // 2, w.cp, -1), s.view(2, w.tokens // 2, w.cp, -1), ws, r, w.cp)
+            for r, (o, s) in enumerate(zip(ins_o, ins_s))]
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(ins_o, ins_s, [o[0] for o in outs], [o[1] for o in outs], with_numpy=False)
+
+
+def test_per_rank_call_twice_is_an_error(hx, ops):
+    cp = 2
+    ws = get_workspace(hx, cp)
+    o = torch.zeros(2, cp, 64, dtype=torch.bfloat16, device="cuda")
+    s = torch.zeros(2, cp, 2, device="cuda")
+    hx.alltoall(o, s, ws, 0, cp)
+    with pytest.raises(RuntimeError, match="again"):
+        hx.alltoall(o, s, ws, 0, cp)
+    hx.alltoall(o, s, ws, 1, cp)  # completes the group
+    torch.cuda.synchronize()
+    assert_clean(ops)
+
+
+# ---------------------------------------------------------------------------
+# what the sender leaves in the FIFO
+# ---------------------------------------------------------------------------
+
+def test_fifo_image_matches_host_model(hx, ops, host_model):
+    import ctypes
+
+    cp, entries, x, s = 2, 300, 512, 8  # 9-line messages, 113 per FIFO entry: 3 entries per stream on one channel
+    cu = torch.cuda.get_device_properties(0).multi_processor_count
+    ws = get_workspace(hx, cp, fresh=True)
+    g = torch.Generator().manual_seed(5)
+    ins_o = [torch.randint(-32768, 32767, (entries, cp, x), generator=g, dtype=torch.int16) for _ in range(cp)]
+    ins_s = [torch.randint(-2**31, 2**31 - 1, (entries, cp, s), generator=g, dtype=torch.int32) for _ in range(cp)]
+    dev_o = [t.view(torch.bfloat16).cuda() for t in ins_o]
+    dev_s = [t.view(torch.float32).cuda() for t in ins_s]
+    out_o = [torch.empty_like(t) for t in dev_o]
+    out_s = [torch.empty_like(t) for t in dev_s]
+    arr = (ops._Params * cp)()
+    for r in range(cp):
+        arr[r] = ops._make_params(dev_o[r], dev_s[r], out_o[r], out_s[r], ws, r, cp, 1)
+    ops._check(ops._lib.helix_a2a_alltoall_send(arr, cp, ops._stream_handle()), "send")
+    torch.cuda.synchronize()
+    assert_clean(ops)
+
+    host_ws = host_model.new_workspace(cp, cu)
+    np_o = [t.numpy().view(np.uint16) for t in ins_o]
+    np_s = [t.numpy().view(np.uint32) for t in ins_s]
+    _, _, rc, msg = host_model.alltoall(np_o, np_s, host_ws, cu, 1, send=True, recv=False)
+    assert rc == 0, msg
+    max_ch = host_model.max_channel_count(cp, cu)
+    fifo_region_elems = FIFO_BYTES * cp * max_ch // 8
+    for row in range(cp):
+        for sender in range(cp):
+            off = host_model.lib.hm_fifo_offset(sender, 0, max_ch) // 8
+            got = ws[row, off: off + FIFO_BYTES // 8].cpu().numpy()
+            assert np.array_equal(got, host_ws[row, off: off + FIFO_BYTES // 8]), f"FIFO {sender}->{row} differs"
+        assert np.array_equal(ws[row, fifo_region_elems:].cpu().numpy(), host_ws[row, fifo_region_elems:])
+    # finish the exchange so the workspace is consistent again
+    ops._check(ops._lib.helix_a2a_alltoall_recv(arr, cp, ops._stream_handle()), "recv")
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(dev_o, dev_s, out_o, out_s)
+
+
+# ---------------------------------------------------------------------------
+# bounded waits and back-pressure
+# ---------------------------------------------------------------------------
+
+def test_receive_without_send_times_out_cleanly(hx, ops):
+    cp = 2
+    ws = get_workspace(hx, cp, fresh=True)
+    o = [torch.zeros(3, cp, 64, dtype=torch.bfloat16, device="cuda") for _ in range(cp)]
+    s = [torch.zeros(3, cp, 2, device="cuda") for _ in range(cp)]
+    out_o = [torch.empty_like(t) for t in o]
+    out_s = [torch.empty_like(t) for t in s]
+    arr = (ops._Params * cp)()
+    for r in range(cp):
+        arr[r] = ops._make_params(o[r], s[r], out_o[r], out_s[r], ws, r, cp, 1)
+    ops.set_spin_limit_us(0)  # every wait gives up at its first clock check: the kernel still exits normally
+    try:
+        ops._check(ops._lib.helix_a2a_alltoall_recv(arr, cp, ops._stream_handle()), "recv")
+        torch.cuda.synchronize()
+        status = ops.device_status()
+    finally:
+        ops.set_spin_limit_us(2_000_000)
+    assert status & 1, "the receiver should have reported a timed-out wait"
+    assert ops.device_status() == 0  # reading clears it
+    for r in range(cp):
+        hx.init_workspace(ws, r, cp)
+
+
+def test_send_capacity_is_checked_for_split_phases(hx, ops):
+    # 2-line messages on one channel: 2048 fit the four FIFO entries; a send-only launch of more is refused
+    cp, entries = 2, 2049
+    ws = get_workspace(hx, cp)
+    o = torch.zeros(entries, cp, 64, dtype=torch.bfloat16, device="cuda")
+    s = torch.zeros(entries, cp, 2, device="cuda")
+    os.environ["HELIX_A2A_CHANNEL_COUNT"] = "1"
+    try:
+        with pytest.raises(RuntimeError, match="FIFO entries in flight"):
+            hx.alltoall(o, s, ws, 0, cp)
+    finally:
+        del os.environ["HELIX_A2A_CHANNEL_COUNT"]
+    ops.reset_logical_ranks()
+
+
+@pytest.mark.parametrize("single_round", [False, True])
+def test_traffic_beyond_fifo_capacity(hx, ops, single_round):
+    # 5000 two-line messages per stream on one channel = 10 FIFO entries. Default: three stream-ordered
+    # rounds. single_round: one launch, senders wait in-kernel until receivers release entries.
+    cp, entries = 2, 5000
+    ws = get_workspace(hx, cp, fresh=True)
+    g = torch.Generator().manual_seed(9)
+    ins_o = [torch.randint(-32768, 32767, (entries, cp, 64), generator=g, dtype=torch.int16).view(torch.bfloat16).cuda()
+             for _ in range(cp)]
+    ins_s = [torch.randn(entries, cp, 2, generator=g).cuda() for _ in range(cp)]
+    ops.set_single_round(single_round)
+    try:
+        outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws, channel_count=1)
+        torch.cuda.synchronize()
+    finally:
+        ops.set_single_round(False)
+    assert_clean(ops)
+    check_against_oracle(ins_o, ins_s, outs_o, outs_s)

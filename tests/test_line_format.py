@@ -1,0 +1,154 @@
+"""CPU checks of the build's own LL128 line format and workspace geometry.
+
+They run the bounds-checked host walk-through of the GPU wave programs
+(tests/host_model, built on csrc/helix_ll128.hpp) and compare its result with
+the oracle, and they inspect the FIFO image it leaves behind.
+"""
+import numpy as np
+import pytest
+
+from helix_testing import FIFO_BYTES, FIFO_ENTRY_BYTES, INFO_BYTES, coded_inputs, random_inputs
+from oracle import helix_oracle as ho
+
+CU = 8  # a small device: 4 channels at cp <= 8 keeps host workspaces small
+
+
+def _exchange(host_model, ins_o, ins_s, channels, cu=CU, ws=None):
+    cp = len(ins_o)
+    ws = ws if ws is not None else host_model.new_workspace(cp, cu)
+    out_o, out_s, rc, msg = host_model.alltoall(ins_o, ins_s, ws, cu, channels)
+    assert rc == 0, msg
+    return out_o, out_s, ws
+
+
+@pytest.mark.parametrize("cp,entries,x,s,channels", [
+    (2, 8, 512, 8, 4),     # 1056-byte payload: 8.8 lines
+    (2, 8, 512, 8, 1),
+    (4, 64, 64, 2, 3),     # per-head layout, 136-byte payload: 2 lines, the second nearly empty
+    (8, 5, 1024, 16, 4),   # 2112 bytes: 17.6 lines
+    (4, 37, 576, 12, 4),   # 1200 bytes: exactly 10 lines
+    (4, 37, 48, 2, 2),     # 104 bytes: less than one line
+    (3, 11, 8, 6, 1),      # 40 bytes, odd cp, stats not a multiple of 16 bytes
+    (1, 9, 64, 2, 2),
+    (16, 3, 256, 4, 2),
+    (2, 2, 8192, 32, 1),   # 16512 bytes: 138 lines
+])
+def test_host_model_matches_oracle(host_model, cp, entries, x, s, channels):
+    ins_o, ins_s = random_inputs(cp, entries, x, s, seed=cp + entries + x)
+    out_o, out_s, _ = _exchange(host_model, ins_o, ins_s, channels)
+    want_o, want_s = ho.exchange_closed_form(ins_o), ho.exchange_closed_form(ins_s)
+    for r in range(cp):
+        assert (out_o[r] == want_o[r]).all()
+        assert (out_s[r] == want_s[r]).all()
+
+
+def test_host_model_matches_reference_model(host_model, ref_model):
+    # same inputs through the reference algorithm (its own wire format) and through this build's
+    ins_o, ins_s = coded_inputs(cp=4, entries=6, x=64, s=4)
+    out_o, out_s, _ = _exchange(host_model, ins_o, ins_s, channels=2)
+    ws = ref_model.new_workspace(4, 8)
+    for r in range(4):
+        ref_model.init_workspace(ws, r, 4, 8)
+    ref_o, ref_s = ref_model.alltoall_all_ranks(ins_o, ins_s, ws, sm_count=8)
+    for r in range(4):
+        assert (out_o[r] == ref_o[r]).all() and (out_s[r] == ref_s[r]).all()
+
+
+def test_line_layout_in_fifo(host_model):
+    # one message of 1056 bytes = 132 pieces -> 9 lines; look at what the sender wrote
+    cp, entries, x, s = 2, 1, 512, 8
+    ins_o, ins_s = random_inputs(cp, entries, x, s, seed=1)
+    ws = host_model.new_workspace(cp, CU)
+    _, _, rc, msg = host_model.alltoall(ins_o, ins_s, ws, CU, 1, send=True, recv=False)
+    assert rc == 0, msg
+    max_ch = host_model.max_channel_count(cp, CU)
+    assert host_model.lib.hm_msg_lines(2 * x, 4 * s) == 9
+    for sender in range(cp):
+        for receiver in range(cp):
+            off = host_model.lib.hm_fifo_offset(sender, 0, max_ch)
+            assert off == (sender * max_ch) * FIFO_BYTES
+            fifo = ws[receiver].view(np.uint64)[off // 8: (off + FIFO_BYTES) // 8]
+            lines = fifo[: 9 * 16].reshape(9, 16)
+            payload = np.concatenate([ins_o[sender][0, receiver].view(np.uint64), ins_s[sender][0, receiver].view(np.uint64)])
+            assert payload.size == 132
+            padded = np.zeros(9 * 15, dtype=np.uint64)
+            padded[:132] = payload
+            assert (lines[:, :15] == padded.reshape(9, 15)).all()   # 15 payload words per line, in order
+            assert (lines[:, 15] == 0).all()                        # flag word = step 0 of a fresh workspace
+            assert (fifo[9 * 16:] == np.uint64(0xFFFFFFFFFFFFFFFF)).all()  # nothing else was touched
+    # counters: each sender stream consumed one FIFO entry; the receiver has not run
+    fifo_region = FIFO_BYTES * cp * max_ch
+    for sender in range(cp):
+        for receiver in range(cp):
+            so = host_model.lib.hm_sender_info_offset(cp, max_ch, receiver, 0)
+            assert so == fifo_region + (receiver * max_ch) * INFO_BYTES
+            head, tail = ws[sender][so // 8], ws[sender][so // 8 + 1]
+            assert (head, tail) == (1, 0)
+            ro = host_model.lib.hm_receiver_info_offset(cp, max_ch, sender, 0)
+            assert ro == fifo_region + INFO_BYTES * cp * max_ch + (sender * max_ch) * INFO_BYTES
+            assert ws[receiver][ro // 8 + 1] == 0
+
+
+def test_unit_to_piece_map_covers_every_piece_once(host_model):
+    for lines in (1, 2, 9, 18, 138):
+        seen = []
+        for g in range(8 * lines):
+            p0 = host_model.lib.hm_unit_first_piece(g)
+            seen.append(p0)
+            if g % 8 != 7:
+                seen.append(p0 + 1)
+        assert seen == list(range(15 * lines))
+
+
+def test_repeated_calls_reuse_entries_with_new_steps(host_model):
+    cp = 2
+    ws = host_model.new_workspace(cp, CU)
+    for call in range(9):
+        ins_o, ins_s = random_inputs(cp, 5, 64, 2, seed=call)
+        out_o, out_s, _ = _exchange(host_model, ins_o, ins_s, channels=2, ws=ws)
+        want_o, want_s = ho.exchange_closed_form(ins_o), ho.exchange_closed_form(ins_s)
+        for r in range(cp):
+            assert (out_o[r] == want_o[r]).all() and (out_s[r] == want_s[r]).all()
+    max_ch = host_model.max_channel_count(cp, CU)
+    so = host_model.lib.hm_sender_info_offset(cp, max_ch, 1, 1)
+    assert ws[0][so // 8] == 9 and ws[0][so // 8 + 1] == 9  # one entry per call and stream
+    # the flag of the first line of FIFO entry 9 % 4 == 1 ... entry 0 was last written at step 8
+    off = host_model.lib.hm_fifo_offset(0, 1, max_ch)
+    fifo = ws[1].view(np.uint64)[off // 8: (off + FIFO_BYTES) // 8]
+    assert fifo[15] == 8
+    assert fifo[FIFO_ENTRY_BYTES // 8 + 15] == 5
+
+
+def test_rounds_when_traffic_exceeds_the_fifo(host_model):
+    # 2-line messages, one channel: 512 messages per entry, 2048 per round; 5000 entries need 3 rounds
+    cp, entries = 2, 5000
+    ins_o, ins_s = random_inputs(cp, entries, 64, 2, seed=7)
+    out_o, out_s, ws = _exchange(host_model, ins_o, ins_s, channels=1)
+    want_o, want_s = ho.exchange_closed_form(ins_o), ho.exchange_closed_form(ins_s)
+    for r in range(cp):
+        assert (out_o[r] == want_o[r]).all() and (out_s[r] == want_s[r]).all()
+    so = host_model.lib.hm_sender_info_offset(cp, host_model.max_channel_count(cp, CU), 0, 0)
+    assert ws[0][so // 8] == 4 + 4 + 2  # entries consumed: 2048 + 2048 + 904 messages
+
+
+def test_receiver_rejects_stale_lines(host_model):
+    # a receive without the matching send must find no valid flag (fresh FIFO holds all ones)
+    cp = 2
+    ins_o, ins_s = random_inputs(cp, 3, 64, 2, seed=2)
+    ws = host_model.new_workspace(cp, CU)
+    _, _, rc, msg = host_model.alltoall(ins_o, ins_s, ws, CU, 1, send=False, recv=True)
+    assert rc > 0 and "flag" in msg
+
+
+def test_bounds_checker_catches_short_buffers(host_model):
+    # the walk-through refuses an access outside its buffer instead of performing it:
+    # a workspace laid out for 4 channels, addressed as if it had 8
+    cp = 2
+    ins_o, ins_s = random_inputs(cp, 4, 64, 2, seed=3)
+    ws = host_model.new_workspace(cp, CU)
+    _, _, rc, _ = host_model.alltoall(ins_o, ins_s, ws, 2 * CU, 4)
+    assert rc > 0 and host_model.lib.hm_last_out_of_extent() > 0
+    # and is silent for the layout it was made for
+    ws = host_model.new_workspace(cp, CU)
+    _, _, rc, _ = host_model.alltoall(ins_o, ins_s, ws, CU, 4)
+    assert rc == 0 and host_model.lib.hm_last_out_of_extent() == 0
