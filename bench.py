@@ -109,6 +109,8 @@ def main() -> int:
     ap.add_argument("--channels", type=int, default=0, help="0 = automatic")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
+                    help="also run 5 elementwise copies (read MIB, write MIB) so that a counter run can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs all context-parallel ranks as logical ranks of ONE GPU; "
@@ -163,6 +165,15 @@ def main() -> int:
         for r in range(w.cp):
             ok &= torch.equal(outs_o[r].view(torch.int16), want_o[r].view(torch.int16))
             ok &= torch.equal(outs_s[r].view(torch.int32), want_s[r].view(torch.int32))
+
+    if args.copy_calibration:
+        n = args.copy_calibration * (1 << 20) // 4
+        src = torch.arange(n, dtype=torch.int32, device="cuda")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(5):
+            torch.add(src, 1, out=dst)  # one kernel: reads 4n bytes, writes 4n bytes
+        torch.cuda.synchronize()
 
     achieved = bytes_per_call / (avg_kernel_ms * 1e-3) / 1e9
     result = {
