@@ -242,6 +242,12 @@ int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs,
   a.sendStride1 = p0.send_fields[1].stride_bytes;
   a.recvStride0 = p0.recv_fields[0].stride_bytes;
   a.recvStride1 = p0.recv_fields[1].stride_bytes;
+  const uint64_t rows = static_cast<uint64_t>(p0.entry_count) * cp;
+  a.sendBytes0 = static_cast<uint32_t>(rows * a.sendStride0);
+  a.sendBytes1 = static_cast<uint32_t>(rows * a.sendStride1);
+  a.recvBytes0 = static_cast<uint32_t>(rows * a.recvStride0);
+  a.recvBytes1 = static_cast<uint32_t>(rows * a.recvStride1);
+  a.lineMagic = line_div_magic(sh.lines);
   a.rankBegin = p0.cp_rank;
   a.rankCount = count;
   a.spinLimitTicks = g_spinLimitUs.load() * 100ull;

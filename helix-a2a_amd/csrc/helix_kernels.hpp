@@ -30,6 +30,9 @@ struct KernelArgs {
   int field0Bytes, field1Bytes;
   int sendStride0, sendStride1;  // bytes between consecutive (entry, peer) rows
   int recvStride0, recvStride1;
+  uint32_t sendBytes0, sendBytes1;  // extent of each tensor (< 2 GiB), the range of its buffer descriptor
+  uint32_t recvBytes0, recvBytes1;
+  uint32_t lineMagic;               // line_div_magic(lines per message)
   int rankBegin, rankCount;
   int doSend, doRecv;
   uint64_t spinLimitTicks;  // bound of one in-kernel wait, in 100 MHz ticks
@@ -39,7 +42,9 @@ struct KernelArgs {
   int statsMode, dtype;
 };
 
-constexpr int kWavesPerBlock = 4;
+// Wavefronts of a workgroup are independent (no LDS, no barrier); small
+// workgroups dispatch and retire at a finer grain (2 measured best of 1..16).
+constexpr int kWavesPerBlock = 2;
 constexpr int kBlockThreads = kWavesPerBlock * kWaveLanes;
 
 // wavefronts one direction of a launch needs: one per (local rank, channel, peer)

@@ -171,6 +171,35 @@ HELIX_HD int cursor_entry_index(const FifoCursor& c) {
   return static_cast<int>(c.step & (kFifoDepth - 1));
 }
 
+// Division of a line index x < 1024 by the lines-per-message count L <= 1024
+// without an integer divide: floor(x / L) == (x * M) >> 20 with
+// M = ceil(2^20 / L). Exact on that range: the excess x * (M - 2^20/L) / 2^20
+// stays below 2^-10 <= 1/L (and is zero for L = 1024).
+constexpr int kLineDivShift = 20;
+HELIX_HD uint32_t line_div_magic(int lines) {
+  return static_cast<uint32_t>(((1u << kLineDivShift) + lines - 1) / lines);
+}
+HELIX_HD uint32_t line_div(uint32_t x, uint32_t magic) { return (x * magic) >> kLineDivShift; }
+
+// Where unit U of a run lives. A run is the sequence of messages a stream
+// puts into one FIFO entry; it starts at line 0 of the entry and its messages
+// follow each other without gaps, so unit U sits at byte U*16 of the entry.
+struct RunUnit {
+  uint32_t msg;     // message index inside the run
+  uint32_t piece0;  // first payload piece of the unit inside its message
+  bool flag;        // second word of the unit is the flag word
+};
+HELIX_HD RunUnit decode_run_unit(uint32_t U, uint32_t lines, uint32_t magic) {
+  RunUnit d;
+  uint32_t x = U >> 3;
+  uint32_t u = U & 7u;
+  d.msg = line_div(x, magic);
+  uint32_t line = x - d.msg * lines;
+  d.piece0 = line * kPiecesPerLine + 2u * u;
+  d.flag = u == 7u;
+  return d;
+}
+
 // Number of FIFO entries a stream of `msgs` messages consumes in one call.
 HELIX_HD int entries_for_msgs(int msgs, const MsgShape& s) {
   if (msgs <= 0) return 0;

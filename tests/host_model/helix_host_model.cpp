@@ -54,7 +54,31 @@ Extent field_extent(const helix_a2a_field_t& f, int entries, int cp) {
   return Extent{static_cast<const uint8_t*>(f.data), static_cast<uint64_t>(entries) * cp * f.stride_bytes};
 }
 
-// sender wave of stream (s -> r, ch)
+// Offsets of the two payload pieces of run unit U, computed in 32-bit
+// arithmetic exactly as the kernels do; kNone where the piece is not in that field.
+constexpr uint32_t kNone = 0x80000000u;
+struct UnitOffsets {
+  uint32_t a0, b0, a1, b1;
+  bool flag;
+};
+
+UnitOffsets unit_offsets(const Ctx& c, uint32_t firstRow, uint32_t rowStep, uint32_t stride0, uint32_t stride1,
+                         uint32_t firstMsg, uint32_t U) {
+  RunUnit d = decode_run_unit(U, static_cast<uint32_t>(c.sh.lines), line_div_magic(c.sh.lines));
+  uint32_t row = firstRow + (firstMsg + d.msg) * rowStep;
+  uint32_t base0 = row * stride0, base1 = row * stride1;
+  uint32_t np0 = static_cast<uint32_t>(c.sh.np0), np = static_cast<uint32_t>(c.sh.np);
+  uint32_t pa = d.piece0, pb = d.piece0 + 1;
+  UnitOffsets o;
+  o.flag = d.flag;
+  o.a0 = pa < np0 ? base0 + pa * kPieceBytes : kNone;
+  o.b0 = (!d.flag && pb < np0) ? base0 + pb * kPieceBytes : kNone;
+  o.a1 = (pa >= np0 && pa < np) ? base1 + (pa - np0) * kPieceBytes : kNone;
+  o.b1 = (!d.flag && pb >= np0 && pb < np) ? base1 + (pb - np0) * kPieceBytes : kNone;
+  return o;
+}
+
+// sender wave of stream (s -> r, ch): one run per FIFO entry, units walked flat
 void run_sender(Ctx& c, int s, int r, int ch) {
   const helix_a2a_params_t& p = c.ranks[s];
   uint8_t* wsBase = reinterpret_cast<uint8_t*>(p.workspace);
@@ -67,45 +91,42 @@ void run_sender(Ctx& c, int s, int r, int ch) {
   Extent fifoExt{fifo, kFifoBytes};
   Extent e0 = field_extent(p.send_fields[0], p.entry_count, c.cp);
   Extent e1 = field_extent(p.send_fields[1], p.entry_count, c.cp);
-  FifoCursor cur = make_cursor(info[0]);
-  for (int e = c.entryBegin + ch; e < c.entryEnd; e += c.channels) {
-    if (cursor_needs_new_entry(cur, c.sh.lines)) {
-      bool closed;
-      cursor_open_entry(cur, &closed);
-      if (closed) info[0] = cur.step;
-      // the model runs senders to completion first: room must already be there
-      if (info[1] + kFifoDepth <= cur.step) {
-        c.chk.violations++;
-        snprintf(c.chk.first, sizeof(c.chk.first), "sender %d->%d ch %d would block at step %lld", s, r, ch,
-                 (long long)cur.step);
-        return;
-      }
+  const int msgs = stream_msg_count(c.entryBegin, c.entryEnd, ch, c.channels);
+  if (msgs == 0) return;
+  const int perEntry = msgs_per_fifo_entry(c.sh);
+  const uint32_t firstRow = static_cast<uint32_t>(c.entryBegin + ch) * c.cp + r;
+  const uint32_t rowStep = static_cast<uint32_t>(c.channels) * c.cp;
+  int64_t step = info[0];
+  for (int firstMsg = 0; firstMsg < msgs; firstMsg += perEntry) {
+    int runMsgs = perEntry < msgs - firstMsg ? perEntry : msgs - firstMsg;
+    uint32_t runUnits = static_cast<uint32_t>(runMsgs) * c.sh.units;
+    if (firstMsg > 0) {
+      step += 1;
+      info[0] = step;
     }
-    uint64_t row = static_cast<uint64_t>(e) * c.cp + r;
-    const uint8_t* row0 = e0.base + row * p.send_fields[0].stride_bytes;
-    const uint8_t* row1 = e1.base + row * p.send_fields[1].stride_bytes;
-    uint32_t msgOff = fifo_unit_offset(cursor_entry_index(cur), cur.lineBase, 0);
-    for (int g = 0; g < c.sh.units; ++g) {  // every lane of every wave access
+    // the model runs senders to completion first: room must already be there
+    if (info[1] + kFifoDepth <= step) {
+      c.chk.violations++;
+      snprintf(c.chk.first, sizeof(c.chk.first), "sender %d->%d ch %d would block at step %lld", s, r, ch,
+               (long long)step);
+      return;
+    }
+    uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
+    for (uint32_t U = 0; U < runUnits; ++U) {  // every lane of every wave access
+      UnitOffsets o = unit_offsets(c, firstRow, rowStep, p.send_fields[0].stride_bytes, p.send_fields[1].stride_bytes,
+                                   firstMsg, U);
       uint64_t words[2] = {0, 0};
-      int p0 = unit_first_piece(g);
+      const uint32_t offs0[2] = {o.a0, o.b0}, offs1[2] = {o.a1, o.b1};
       for (int k = 0; k < 2; ++k) {
-        int piece = p0 + k;
-        if (k == 1 && unit_has_flag(g)) {
-          words[1] = static_cast<uint64_t>(cur.step);
-        } else if (piece < c.sh.np0) {
-          const uint8_t* src = row0 + piece * kPieceBytes;
-          if (c.chk.ok(e0, src, 8, "send field 0")) memcpy(&words[k], src, 8);
-        } else if (piece < c.sh.np) {
-          const uint8_t* src = row1 + (piece - c.sh.np0) * kPieceBytes;
-          if (c.chk.ok(e1, src, 8, "send field 1")) memcpy(&words[k], src, 8);
-        }
+        if (offs0[k] != kNone && c.chk.ok(e0, e0.base + offs0[k], 8, "send field 0")) memcpy(&words[k], e0.base + offs0[k], 8);
+        if (offs1[k] != kNone && c.chk.ok(e1, e1.base + offs1[k], 8, "send field 1")) memcpy(&words[k], e1.base + offs1[k], 8);
       }
-      uint8_t* dst = fifo + msgOff + g * kUnitBytes;
+      if (o.flag) words[1] = static_cast<uint64_t>(step);
+      uint8_t* dst = fifo + entryOffset + U * kUnitBytes;
       if (c.chk.ok(fifoExt, dst, 16, "fifo store")) memcpy(dst, words, 16);
     }
-    cur.lineBase += c.sh.lines;
   }
-  if (cur.open) info[0] = cur.step + 1;
+  info[0] = step + 1;
 }
 
 // receiver wave of stream (s -> r, ch); a line whose flag is not there counts as a violation
@@ -124,53 +145,47 @@ void run_receiver(Ctx& c, int r, int s, int ch) {
   Extent fifoExt{fifo, kFifoBytes};
   Extent e0 = field_extent(p.recv_fields[0], p.entry_count, c.cp);
   Extent e1 = field_extent(p.recv_fields[1], p.entry_count, c.cp);
-  FifoCursor cur = make_cursor(info[1]);
-  for (int e = c.entryBegin + ch; e < c.entryEnd; e += c.channels) {
-    if (cursor_needs_new_entry(cur, c.sh.lines)) {
-      bool closed;
-      cursor_open_entry(cur, &closed);
-      if (closed) {
-        info[1] = cur.step;
-        sinfo[1] = cur.step;
-      }
+  const int msgs = stream_msg_count(c.entryBegin, c.entryEnd, ch, c.channels);
+  if (msgs == 0) return;
+  const int perEntry = msgs_per_fifo_entry(c.sh);
+  const uint32_t firstRow = static_cast<uint32_t>(c.entryBegin + ch) * c.cp + s;
+  const uint32_t rowStep = static_cast<uint32_t>(c.channels) * c.cp;
+  int64_t step = info[1];
+  for (int firstMsg = 0; firstMsg < msgs; firstMsg += perEntry) {
+    int runMsgs = perEntry < msgs - firstMsg ? perEntry : msgs - firstMsg;
+    uint32_t runUnits = static_cast<uint32_t>(runMsgs) * c.sh.units;
+    if (firstMsg > 0) {
+      step += 1;
+      info[1] = step;
+      sinfo[1] = step;
     }
-    uint64_t row = static_cast<uint64_t>(e) * c.cp + s;
-    uint8_t* row0 = const_cast<uint8_t*>(e0.base) + row * p.recv_fields[0].stride_bytes;
-    uint8_t* row1 = const_cast<uint8_t*>(e1.base) + row * p.recv_fields[1].stride_bytes;
-    uint32_t msgOff = fifo_unit_offset(cursor_entry_index(cur), cur.lineBase, 0);
-    for (int g = 0; g < c.sh.units; ++g) {
-      const uint8_t* src = fifo + msgOff + g * kUnitBytes;
+    uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
+    for (uint32_t U = 0; U < runUnits; ++U) {
+      const uint8_t* src = fifo + entryOffset + U * kUnitBytes;
       if (!c.chk.ok(fifoExt, src, 16, "fifo load")) continue;
       uint64_t words[2];
       memcpy(words, src, 16);
-      // flag of this lane's line
-      uint64_t flag;
-      memcpy(&flag, fifo + msgOff + (g | 7) * kUnitBytes + 8, 8);
-      if (flag != static_cast<uint64_t>(cur.step)) {
+      uint64_t flag;  // flag of this lane's line
+      memcpy(&flag, fifo + entryOffset + (U | 7u) * kUnitBytes + 8, 8);
+      if (flag != static_cast<uint64_t>(step)) {
         if (c.chk.violations++ == 0)
-          snprintf(c.chk.first, sizeof(c.chk.first), "stream %d->%d ch %d entry %d: flag %llx != step %llx", s, r, ch,
-                   e, (unsigned long long)flag, (unsigned long long)cur.step);
+          snprintf(c.chk.first, sizeof(c.chk.first), "stream %d->%d ch %d unit %u: flag %llx != step %llx", s, r, ch, U,
+                   (unsigned long long)flag, (unsigned long long)step);
         continue;
       }
-      int p0 = unit_first_piece(g);
+      UnitOffsets o = unit_offsets(c, firstRow, rowStep, p.recv_fields[0].stride_bytes, p.recv_fields[1].stride_bytes,
+                                   firstMsg, U);
+      const uint32_t offs0[2] = {o.a0, o.b0}, offs1[2] = {o.a1, o.b1};
+      uint8_t* base0 = const_cast<uint8_t*>(e0.base);
+      uint8_t* base1 = const_cast<uint8_t*>(e1.base);
       for (int k = 0; k < 2; ++k) {
-        int piece = p0 + k;
-        if (k == 1 && unit_has_flag(g)) break;
-        if (piece < c.sh.np0) {
-          uint8_t* dst = row0 + piece * kPieceBytes;
-          if (c.chk.ok(e0, dst, 8, "recv field 0")) memcpy(dst, &words[k], 8);
-        } else if (piece < c.sh.np) {
-          uint8_t* dst = row1 + (piece - c.sh.np0) * kPieceBytes;
-          if (c.chk.ok(e1, dst, 8, "recv field 1")) memcpy(dst, &words[k], 8);
-        }
+        if (offs0[k] != kNone && c.chk.ok(e0, base0 + offs0[k], 8, "recv field 0")) memcpy(base0 + offs0[k], &words[k], 8);
+        if (offs1[k] != kNone && c.chk.ok(e1, base1 + offs1[k], 8, "recv field 1")) memcpy(base1 + offs1[k], &words[k], 8);
       }
     }
-    cur.lineBase += c.sh.lines;
   }
-  if (cur.open) {
-    info[1] = cur.step + 1;
-    sinfo[1] = cur.step + 1;
-  }
+  info[1] = step + 1;
+  sinfo[1] = step + 1;
 }
 
 }  // namespace
@@ -230,5 +245,14 @@ uint64_t hm_receiver_info_offset(int cp, int max_ch, int sender, int channel) {
 }
 int hm_msg_lines(int f0, int f1) { return make_msg_shape(f0, f1).lines; }
 int hm_unit_first_piece(int g) { return unit_first_piece(g); }
+// floor(x / lines) the way the kernels compute it
+uint32_t hm_line_div(uint32_t x, int lines) { return line_div(x, line_div_magic(lines)); }
+// number of line indices x of a FIFO entry for which that differs from x / lines
+int hm_line_div_mismatches(int lines) {
+  int bad = 0;
+  for (uint32_t x = 0; x < static_cast<uint32_t>(kFifoEntryLines); ++x)
+    bad += line_div(x, line_div_magic(lines)) != x / static_cast<uint32_t>(lines);
+  return bad;
+}
 
 }  // extern "C"

@@ -100,6 +100,13 @@ def test_unit_to_piece_map_covers_every_piece_once(host_model):
         assert seen == list(range(15 * lines))
 
 
+def test_line_division_is_exact(host_model):
+    # the multiply-shift that replaces x / lines must be exact for every line index of a FIFO entry
+    for lines in range(1, 1025):
+        assert host_model.lib.hm_line_div_mismatches(lines) == 0, lines
+    assert [host_model.lib.hm_line_div(x, 18) for x in (0, 17, 18, 35, 36, 1007, 1023)] == [0, 0, 1, 1, 2, 55, 56]
+
+
 def test_repeated_calls_reuse_entries_with_new_steps(host_model):
     cp = 2
     ws = host_model.new_workspace(cp, CU)
