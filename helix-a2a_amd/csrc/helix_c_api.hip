@@ -240,8 +240,8 @@ int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs,
   a.field1Bytes = f1;
   a.sendStride0 = p0.send_fields[0].stride_bytes;
   a.sendStride1 = p0.send_fields[1].stride_bytes;
-  a.recvStride0 = p0.recv_fields[0].stride_bytes;
-  a.recvStride1 = p0.recv_fields[1].stride_bytes;
+  a.recvStride0 = exchangeOutputs ? p0.recv_fields[0].stride_bytes : 0;
+  a.recvStride1 = exchangeOutputs ? p0.recv_fields[1].stride_bytes : 0;
   const uint64_t rows = static_cast<uint64_t>(p0.entry_count) * cp;
   a.sendBytes0 = static_cast<uint32_t>(rows * a.sendStride0);
   a.sendBytes1 = static_cast<uint32_t>(rows * a.sendStride1);
@@ -367,9 +367,55 @@ int helix_a2a_alltoall_loopback(const helix_a2a_params_t* per_rank, int cp_size,
   return launch_rounds(plan, true, true, true, static_cast<hipStream_t>(stream));
 }
 
-int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t*, const helix_a2a_combine_out_t*, int, int, int,
-                                        void*) {
-  return fail(HELIX_A2A_ERR_RUNTIME, "fused combine is not built into this library");
+int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, const helix_a2a_combine_out_t* out,
+                                        int cp_size, int stats_mode, int dtype, void* stream) {
+  if (per_rank == nullptr || out == nullptr)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "no rank descriptors or outputs given");
+  if (per_rank[0].cp_size != cp_size || per_rank[0].cp_rank != 0)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "loopback needs descriptors of ranks 0..cp_size-1 in order");
+  if (stats_mode != HELIX_A2A_STATS_LSE && stats_mode != HELIX_A2A_STATS_MAX_SUM)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "unknown stats_mode %d", stats_mode);
+  if (dtype != HELIX_A2A_DTYPE_BF16 && dtype != HELIX_A2A_DTYPE_FP16)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "unknown dtype %d", dtype);
+  Plan plan;
+  int rc = build_plan(per_rank, cp_size, false, &plan);
+  if (rc) return rc;
+  KernelArgs& a = plan.args;
+  const int x = per_rank[0].send_fields[0].element_count;
+  const int heads = per_rank[0].send_fields[1].element_count / 2;
+  if (heads < 1 || x % heads != 0 || (x / heads) % 4 != 0)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT,
+                "combine needs partial_o rows of heads * head_dim elements with head_dim a multiple of 4 "
+                "(row of %d elements, %d heads)", x, heads);
+  a.heads = heads;
+  a.headDim = x / heads;
+  a.statsMode = stats_mode;
+  a.dtype = dtype;
+  a.headMagic = head_div_magic(static_cast<uint32_t>(a.headDim) * 2u / kPieceBytes);
+  const uint32_t lds = combine_lds_bytes(cp_size, plan.shape, heads);
+  if (lds > 159u * 1024u)
+    return fail(HELIX_A2A_ERR_CAPACITY, "combine needs %u bytes of LDS per workgroup (cp_size x message), more than a CU has", lds);
+  const uint64_t outBytes = static_cast<uint64_t>(plan.entryCount) * a.field0Bytes;
+  if (outBytes >= 2147483648ull) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "combined output exceeds 2 GiB");
+  a.recvBytes0 = static_cast<uint32_t>(outBytes);
+  a.recvBytes1 = static_cast<uint32_t>(static_cast<uint64_t>(plan.entryCount) * heads * 4u);
+  for (int r = 0; r < cp_size; ++r) {
+    if (plan.entryCount > 0 && out[r].combined == nullptr)
+      return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "combined output of rank %d is null", r);
+    if ((reinterpret_cast<uintptr_t>(out[r].combined) % kPieceBytes) != 0 ||
+        (reinterpret_cast<uintptr_t>(out[r].lse_out) % 4) != 0)
+      return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "combine outputs of rank %d are misaligned", r);
+    a.rank[r].recv0 = static_cast<uint8_t*>(out[r].combined);
+    a.rank[r].recv1 = reinterpret_cast<uint8_t*>(out[r].lse_out);
+  }
+  if (plan.entryCount == 0) return HELIX_A2A_OK;
+  for (int begin = 0; begin < plan.entryCount; begin += plan.roundEntries) {
+    a.entryBegin = begin;
+    long end = static_cast<long>(begin) + plan.roundEntries;
+    a.entryEnd = end > plan.entryCount ? plan.entryCount : static_cast<int>(end);
+    HELIX_HIP_TRY(launch_combine(a, static_cast<hipStream_t>(stream)));
+  }
+  return HELIX_A2A_OK;
 }
 
 int helix_a2a_device_status(uint32_t* status, void* stream) {

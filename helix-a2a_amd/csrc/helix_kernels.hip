@@ -26,6 +26,8 @@
 // stream may run on different XCDs).
 #include "helix_kernels.hpp"
 
+#include <hip/hip_fp16.h>
+
 namespace helix {
 namespace {
 
@@ -328,6 +330,214 @@ __global__ __launch_bounds__(kBlockThreads) void helix_exchange_kernel(KernelArg
   }
 }
 
+// ---------------------------------------------------------------------------
+// exchange fused with the LSE-weighted combine
+// ---------------------------------------------------------------------------
+// Element conversions of partial_o (4 elements per 8-byte piece).
+template <int kDtype>
+__device__ __forceinline__ void widen4(u32x2 piece, float (&f)[4]);
+template <>
+__device__ __forceinline__ void widen4<0>(u32x2 piece, float (&f)[4]) {  // bf16: the upper half of an fp32
+  f[0] = __uint_as_float(piece.x << 16);
+  f[1] = __uint_as_float(piece.x & 0xFFFF0000u);
+  f[2] = __uint_as_float(piece.y << 16);
+  f[3] = __uint_as_float(piece.y & 0xFFFF0000u);
+}
+template <>
+__device__ __forceinline__ void widen4<1>(u32x2 piece, float (&f)[4]) {  // fp16
+  f[0] = __half2float(__ushort_as_half(static_cast<unsigned short>(piece.x & 0xFFFFu)));
+  f[1] = __half2float(__ushort_as_half(static_cast<unsigned short>(piece.x >> 16)));
+  f[2] = __half2float(__ushort_as_half(static_cast<unsigned short>(piece.y & 0xFFFFu)));
+  f[3] = __half2float(__ushort_as_half(static_cast<unsigned short>(piece.y >> 16)));
+}
+
+template <int kDtype>
+__device__ __forceinline__ uint32_t narrow1(float v);
+template <>
+__device__ __forceinline__ uint32_t narrow1<0>(float v) {  // fp32 -> bf16, round to nearest even, NaN stays NaN
+  uint32_t b = __float_as_uint(v);
+  if ((b & 0x7FFFFFFFu) > 0x7F800000u) return (b >> 16) | 0x0040u;
+  return (b + 0x7FFFu + ((b >> 16) & 1u)) >> 16;
+}
+template <>
+__device__ __forceinline__ uint32_t narrow1<1>(float v) {
+  return static_cast<uint32_t>(__half_as_ushort(__float2half_rn(v)));
+}
+
+// Receive half of the fused form: the cpSize wavefronts of a workgroup each
+// poll one sender's FIFO for the same (receiver, channel), park the payload
+// pieces in LDS, and the workgroup then reduces over the senders:
+//   out[e, h, :] = sum_s w[s, h] * partial_o_s[e, h, :],  w = softmax_s(lse[s, h])
+// (patches/dcp_alltoall_helix.py:142-207). LDS: [cp][np] pieces, then [cp][heads] weights.
+template <int kDtype>
+__device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r, int s, int ch, int lane,
+                                                     uint8_t* lds, int* failed) {
+  Stream st;
+  setup_stream(st, a, s, ch);
+  if (st.msgs == 0) return;  // uniform over the workgroup: same channel
+  uint8_t* senderRow = a.workspace + static_cast<uint64_t>(s) * a.rowStrideBytes;
+  uint8_t* receiverRow = a.workspace + static_cast<uint64_t>(r) * a.rowStrideBytes;
+  int64_t* senderInfo = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(a.cpSize, a.maxChannels, r, ch));
+  int64_t* info = reinterpret_cast<int64_t*>(receiverRow + receiver_info_offset(a.cpSize, a.maxChannels, s, ch));
+  st.fifo = make_rsrc(receiverRow + fifo_offset(s, ch, a.maxChannels), kFifoBytes);
+  __amdgpu_buffer_rsrc_t outRsrc = make_rsrc(a.rank[r].recv0, a.recvBytes0);
+  float* lseOut = reinterpret_cast<float*>(a.rank[r].recv1);
+
+  u32x2* pieces = reinterpret_cast<u32x2*>(lds);                                    // [cp][np]
+  float* weights = reinterpret_cast<float*>(lds + static_cast<size_t>(a.cpSize) * st.np * kPieceBytes);  // [cp][heads]
+  u32x2* myPieces = pieces + static_cast<size_t>(s) * st.np;
+
+  int64_t step = info[1];
+  const int flagLane = lane | 7;
+  const int tid = static_cast<int>(threadIdx.x);
+  const int threads = static_cast<int>(blockDim.x);
+
+  for (int k = 0; k < st.msgs; ++k) {
+    const int posInRun = k % st.msgsPerEntry;
+    if (k > 0 && posInRun == 0) {
+      step += 1;
+      if (lane == 0) {
+        st_counter(&info[1], step);
+        st_counter(&senderInfo[1], step);
+      }
+    }
+    const uint32_t msgOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes +
+                               static_cast<uint32_t>(posInRun) * st.lines * kLineBytes;
+    const uint32_t stepLo = static_cast<uint32_t>(step);
+    const uint32_t stepHi = static_cast<uint32_t>(static_cast<uint64_t>(step) >> 32);
+    bool timedOut = false;
+    for (uint32_t U0 = 0; U0 < st.unitsPerMsg && !timedOut; U0 += kUnitsInFlight * kWaveLanes) {
+      bool pending[kUnitsInFlight];
+#pragma unroll
+      for (int i = 0; i < kUnitsInFlight; ++i) pending[i] = (U0 + i * kWaveLanes + lane) < st.unitsPerMsg;
+      SpinGuard guard(a.spinLimitTicks);
+      for (;;) {
+        u32x4 v[kUnitsInFlight];
+#pragma unroll
+        for (int i = 0; i < kUnitsInFlight; ++i) {
+          uint32_t U = U0 + i * kWaveLanes + lane;
+          uint32_t off = pending[i] ? msgOffset + U * kUnitBytes : kOutOfRange;
+          v[i] = __builtin_amdgcn_raw_buffer_load_b128(st.fifo, off, 0, kAuxSc1);
+        }
+        bool anyPending = false;
+#pragma unroll
+        for (int i = 0; i < kUnitsInFlight; ++i) {
+          uint32_t U = U0 + i * kWaveLanes + lane;
+          bool isFlagLane = (U & 7u) == 7u;
+          bool ok = !pending[i] || !isFlagLane || (v[i].z == stepLo && v[i].w == stepHi);
+          unsigned long long okMask = __ballot(ok);
+          bool lineOk = (okMask >> flagLane) & 1ull;
+          if (pending[i] && lineOk) {
+            uint32_t pa = static_cast<uint32_t>(unit_first_piece(static_cast<int>(U)));
+            if (pa < st.np) {
+              u32x2 wa = {v[i].x, v[i].y};
+              myPieces[pa] = wa;
+            }
+            if (!isFlagLane && pa + 1 < st.np) {
+              u32x2 wb = {v[i].z, v[i].w};
+              myPieces[pa + 1] = wb;
+            }
+          }
+          pending[i] = pending[i] && !lineOk;
+          anyPending |= pending[i];
+        }
+        if (__ballot(anyPending) == 0ull) break;
+        if (guard.expired()) {
+          timedOut = true;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+        asm volatile("" ::: "memory");
+      }
+    }
+    if (timedOut) {
+      raise_status(a.status, kStatusRecvTimeout, lane);
+      if (lane == 0) atomicOr(failed, 1);
+    }
+    __syncthreads();
+    if (*failed) return;  // every wavefront of the workgroup sees the same value here
+
+    // weights of every (sender, head): softmax over the senders of the log-sum-exp
+    const int entry = a.entryBegin + ch + k * a.runChannels;
+    for (int h = tid; h < a.heads; h += threads) {
+      float lse[kMaxCpSize];
+      float m = -INFINITY;
+#pragma unroll
+      for (int q = 0; q < kMaxCpSize; ++q) {
+        if (q < a.cpSize) {
+          u32x2 st2 = pieces[static_cast<size_t>(q) * st.np + st.np0 + h];  // {stats[2h], stats[2h+1]}
+          float x = __uint_as_float(st2.x);
+          if (a.statsMode == 1) x = x + logf(__uint_as_float(st2.y));   // running max + ln(running sum)
+          if (isnan(x) || isinf(x)) x = -INFINITY;
+          lse[q] = x;
+          m = fmaxf(m, x);
+        }
+      }
+      if (m == -INFINITY) m = 0.0f;
+      float total = 0.0f;
+#pragma unroll
+      for (int q = 0; q < kMaxCpSize; ++q) {
+        if (q < a.cpSize) {
+          float w = expf(lse[q] - m);
+          if (isnan(w)) w = 0.0f;
+          lse[q] = w;
+          total += w;
+        }
+      }
+      float inv = 1.0f / fmaxf(total, 1e-10f);
+#pragma unroll
+      for (int q = 0; q < kMaxCpSize; ++q) {
+        if (q < a.cpSize) weights[q * a.heads + h] = lse[q] * inv;
+      }
+      if (lseOut != nullptr) lseOut[static_cast<size_t>(entry) * a.heads + h] = logf(total) + m;
+    }
+    __syncthreads();
+
+    // weighted sum over the senders, 4 elements (one piece) per thread and step
+    for (uint32_t j = static_cast<uint32_t>(tid); j < st.np0; j += static_cast<uint32_t>(threads)) {
+      uint32_t h = head_of_piece(j, a.headMagic);
+      float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      for (int q = 0; q < a.cpSize; ++q) {
+        float f[4];
+        widen4<kDtype>(pieces[static_cast<size_t>(q) * st.np + j], f);
+        float w = weights[q * a.heads + h];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[c] += w * f[c];
+      }
+      u32x2 o = {narrow1<kDtype>(acc[0]) | (narrow1<kDtype>(acc[1]) << 16),
+                 narrow1<kDtype>(acc[2]) | (narrow1<kDtype>(acc[3]) << 16)};
+      uint32_t off = static_cast<uint32_t>(entry) * (st.np0 * kPieceBytes) + j * kPieceBytes;
+      __builtin_amdgcn_raw_buffer_store_b64(o, outRsrc, off, 0, kAuxNone);
+    }
+    __syncthreads();  // LDS is reused by the next message
+  }
+  if (lane == 0) {
+    st_counter(&info[1], step + 1);
+    st_counter(&senderInfo[1], step + 1);
+  }
+}
+
+// Workgroups of cpSize wavefronts. The first rankCount*runChannels workgroups
+// send (workgroup = (sender, channel), wavefront = receiver), the rest receive
+// and combine (workgroup = (receiver, channel), wavefront = sender).
+template <int kDtype>
+__global__ __launch_bounds__(kMaxCpSize * kWaveLanes) void helix_combine_kernel(KernelArgs a) {
+  extern __shared__ __align__(16) uint8_t dynamicLds[];
+  __shared__ int failed;
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWaveLanes);
+  const int lane = static_cast<int>(threadIdx.x) % kWaveLanes;
+  const int sendBlocks = a.rankCount * a.runChannels;
+  int b = static_cast<int>(blockIdx.x);
+  if (b < sendBlocks) {
+    run_sender<kAuxSc1>(a, a.rankBegin + b / a.runChannels, wave, b % a.runChannels, lane);
+    return;
+  }
+  b -= sendBlocks;
+  if (threadIdx.x == 0) failed = 0;
+  __syncthreads();
+  run_combine_receiver<kDtype>(a, a.rankBegin + b / a.runChannels, wave, b % a.runChannels, lane, dynamicLds, &failed);
+}
+
 // FIFO region <- 0xFF bytes, info regions <- 0 (csrc/helix_alltoall.cu:637-643).
 __global__ __launch_bounds__(256) void helix_init_row_kernel(u32x4* row, uint64_t fifoUnits, uint64_t totalUnits) {
   const u32x4 ones = {0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu};
@@ -349,7 +559,29 @@ hipError_t launch_exchange(const KernelArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_combine_recv(const KernelArgs&, hipStream_t) { return hipErrorNotSupported; }
+hipError_t launch_combine(const KernelArgs& a, hipStream_t stream) {
+  int blocks = 2 * a.rankCount * a.runChannels;
+  if (blocks <= 0) return hipSuccess;
+  const MsgShape sh = make_msg_shape(a.field0Bytes, a.field1Bytes);
+  uint32_t lds = combine_lds_bytes(a.cpSize, sh, a.heads);
+  dim3 block(static_cast<unsigned>(a.cpSize * kWaveLanes));
+  if (a.dtype == 1) {
+    if (lds > 64u * 1024u) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&helix_combine_kernel<1>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+      if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(helix_combine_kernel<1>, dim3(blocks), block, lds, stream, a);
+  } else {
+    if (lds > 64u * 1024u) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&helix_combine_kernel<0>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+      if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(helix_combine_kernel<0>, dim3(blocks), block, lds, stream, a);
+  }
+  return hipGetLastError();
+}
 
 hipError_t launch_init_row(uint8_t* row, uint64_t fifoBytes, uint64_t infoBytes, hipStream_t stream) {
   uint64_t fifoUnits = fifoBytes / kUnitBytes;

@@ -200,6 +200,18 @@ HELIX_HD RunUnit decode_run_unit(uint32_t U, uint32_t lines, uint32_t magic) {
   return d;
 }
 
+// Head index of payload piece p when a head spans `piecesPerHead` pieces
+// (head_dim * 2 bytes / 8): floor(p / piecesPerHead) as a multiply-high by
+// M = floor(2^32 / piecesPerHead) + 1. Exact for p < 2^16 and
+// 2 <= piecesPerHead < 2^16 (the excess p * (M - 2^32/d) / 2^32 is below
+// 2^-16 <= 1/d); piecesPerHead == 1 is the identity and uses magic 0.
+HELIX_HD uint32_t head_div_magic(uint32_t piecesPerHead) {
+  return piecesPerHead <= 1 ? 0u : static_cast<uint32_t>((1ull << 32) / piecesPerHead) + 1u;
+}
+HELIX_HD uint32_t head_of_piece(uint32_t p, uint32_t magic) {
+  return magic == 0u ? p : static_cast<uint32_t>((static_cast<uint64_t>(p) * magic) >> 32);
+}
+
 // Number of FIFO entries a stream of `msgs` messages consumes in one call.
 HELIX_HD int entries_for_msgs(int msgs, const MsgShape& s) {
   if (msgs <= 0) return 0;

@@ -31,6 +31,9 @@ __all__ = [
     "init_workspace",
     "alltoall",
     "alltoall_loopback",
+    "alltoall_combine_loopback",
+    "STATS_LSE",
+    "STATS_MAX_SUM",
 ]
 
 
@@ -105,3 +108,22 @@ def alltoall_loopback(
 ) -> Tuple[List[torch.Tensor], List[torch.Tensor]]:
     """Exchange of all logical ranks in one launch: element ``r`` of each list is rank ``r``."""
     return _ops.alltoall_loopback(partial_o, softmax_stats, workspace, channel_count, out)
+
+
+def alltoall_combine_loopback(
+    partial_o: Sequence[torch.Tensor],
+    softmax_stats: Sequence[torch.Tensor],
+    workspace: torch.Tensor,
+    stats_mode: int = STATS_MAX_SUM,
+    return_lse: bool = False,
+    channel_count: int = 0,
+):
+    """Exchange of all logical ranks fused with the LSE-weighted combine.
+
+    Returns ``combined`` (list, rank ``r`` holds ``[E, heads * head_dim]``) or
+    ``(combined, lse)`` with ``lse[r]`` of shape ``[E, heads]`` when ``return_lse``.
+    ``stats_mode`` says how ``softmax_stats`` pairs encode the weight:
+    ``STATS_LSE`` (slot 0 is the natural-log LSE) or ``STATS_MAX_SUM``
+    (running max, running sum).
+    """
+    return _ops.alltoall_combine_loopback(partial_o, softmax_stats, workspace, stats_mode, return_lse, channel_count)

@@ -380,6 +380,73 @@ class LoopbackPlan:
         return self.out_o, self.out_s
 
 
+class CombinePlan:
+    """Loopback exchange fused with the LSE-weighted combine, replayable with one C call.
+
+    Rank ``r`` ends up with ``combined[r]`` of shape ``[E, heads * head_dim]`` (or
+    ``[E, heads, head_dim]`` for 4-D inputs): for every entry and head the
+    softmax-over-ranks weighted sum of the ``cp_size`` partial outputs it would
+    have received, and optionally ``lse[r]`` ``[E, heads]``, the combined
+    log-sum-exp (the reduction of patches/dcp_alltoall_helix.py:142-207).
+    """
+
+    def __init__(self, partial_o: Sequence[torch.Tensor], softmax_stats: Sequence[torch.Tensor],
+                 workspace: torch.Tensor, stats_mode: int = STATS_MAX_SUM, return_lse: bool = False,
+                 channel_count: int = 0) -> None:
+        cp_size = len(partial_o)
+        _require(1 <= cp_size <= MAX_CP_SIZE and len(softmax_stats) == cp_size,
+                 "need one partial_o and one softmax_stats tensor per rank")
+        _require(stats_mode in (STATS_LSE, STATS_MAX_SUM), "stats_mode must be STATS_LSE or STATS_MAX_SUM")
+        _check_workspace(workspace, cp_size)
+        self.cp_size = cp_size
+        self.inputs = (list(partial_o), list(softmax_stats))
+        self.workspace = workspace
+        self.stats_mode = stats_mode
+        self.combined: List[torch.Tensor] = []
+        self.lse: Optional[List[torch.Tensor]] = [] if return_lse else None
+        self._arr = (_Params * cp_size)()
+        self._out = (_CombineOut * cp_size)()
+        shape0 = None
+        with torch.cuda.device(workspace.device):
+            for r in range(cp_size):
+                o, st = partial_o[r], softmax_stats[r]
+                o3, s3 = _as_3d(o, st, cp_size)
+                sig = (tuple(o3.shape), tuple(s3.shape), o.dtype)
+                shape0 = shape0 or sig
+                _require(sig == shape0, "all ranks must exchange tensors of one shape and dtype")
+                entries, _, x = o3.shape
+                heads = s3.size(-1) // 2
+                _require(x % heads == 0 and (x // heads) % 4 == 0,
+                         "partial_o rows must hold heads * head_dim elements, head_dim a multiple of 4")
+                four_d = o.dim() == 4 and o.size(1) == cp_size and o.size(2) == heads
+                out_shape = (entries, heads, x // heads) if four_d else (entries, x)
+                comb = torch.empty(out_shape, dtype=o.dtype, device=o.device)
+                self.combined.append(comb)
+                self._arr[r] = _make_params(o3, s3, None, None, workspace, r, cp_size, channel_count)
+                self._out[r].combined = comb.data_ptr()
+                if return_lse:
+                    lse = torch.empty(entries, heads, dtype=torch.float32, device=o.device)
+                    self.lse.append(lse)
+                    self._out[r].lse_out = lse.data_ptr()
+                else:
+                    self._out[r].lse_out = None
+        self._dtype = 0 if shape0[2] == torch.bfloat16 else 1
+
+    def run(self):
+        rc = _lib.helix_a2a_alltoall_combine_loopback(self._arr, self._out, self.cp_size, self.stats_mode,
+                                                      self._dtype, _stream_handle())
+        if rc != 0:
+            _raise_last("alltoall_combine_loopback")
+        return (self.combined, self.lse) if self.lse is not None else self.combined
+
+
+def alltoall_combine_loopback(partial_o: Sequence[torch.Tensor], softmax_stats: Sequence[torch.Tensor],
+                              workspace: torch.Tensor, stats_mode: int = STATS_MAX_SUM, return_lse: bool = False,
+                              channel_count: int = 0):
+    """One fused exchange + combine of all logical ranks; see :class:`CombinePlan`."""
+    return CombinePlan(partial_o, softmax_stats, workspace, stats_mode, return_lse, channel_count).run()
+
+
 def device_status() -> int:
     """Read and clear the device status word (synchronises the current stream)."""
     st = ctypes.c_uint32(0)

@@ -1,0 +1,173 @@
+"""GPU tests of the exchange fused with the LSE-weighted combine, against the oracle.
+
+Tolerance: 2e-2 absolute plus 2e-2 relative on the bf16/fp16 result (the oracle
+reduces in fp32 and does not round its result); the combined log-sum-exp is
+fp32 on both sides and is held to 1e-4.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helix_testing import torch_bits
+from oracle import helix_oracle as ho
+
+pytestmark = pytest.mark.gpu
+
+ATOL = RTOL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def hx():
+    import helix_a2a
+
+    assert torch.cuda.is_available()
+    return helix_a2a
+
+
+@pytest.fixture(scope="module")
+def ops(hx):
+    from helix_a2a import _ops
+
+    return _ops
+
+
+_WS = {}
+
+
+def workspace(hx, cp):
+    ws = _WS.get(cp)
+    if ws is None:
+        ws = _WS[cp] = hx.allocate_workspace(cp, 0)
+        for r in range(cp):
+            hx.init_workspace(ws, r, cp)
+    return ws
+
+
+def oracle_combine(ins_o, ins_s, heads, mode, widen):
+    """Exchange (closed form on bits) followed by the reference's combine, per rank."""
+    recv_o = ho.exchange_closed_form([torch_bits(t) for t in ins_o])
+    recv_s = ho.exchange_closed_form([torch_bits(t) for t in ins_s])
+    out = []
+    for r in range(len(ins_o)):
+        o32 = widen(recv_o[r])
+        s32 = recv_s[r].view(np.float32)
+        with np.errstate(all="ignore"):
+            out.append(ho.combine_after_exchange(o32, s32, heads, mode))
+    return out
+
+
+def check(combined, lse, want, dtype):
+    for r, (want_c, want_l) in enumerate(want):
+        got = combined[r].float().cpu().numpy().reshape(want_c.shape)
+        finite = np.isfinite(want_c)
+        assert np.array_equal(np.isfinite(got), finite), f"rank {r}: non-finite pattern differs"
+        err = np.abs(got[finite] - want_c[finite])
+        bound = ATOL + RTOL * np.abs(want_c[finite])
+        assert (err <= bound).all(), f"rank {r}: max error {err.max()} (dtype {dtype})"
+        if lse is not None:
+            g = lse[r].cpu().numpy()
+            inf = np.isneginf(want_l)
+            assert np.array_equal(np.isneginf(g), inf)
+            assert np.allclose(g[~inf], want_l[~inf], rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c5b", "c3", "c4", "c5a"])
+def test_combine_workloads(hx, ops, name):
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS[name]
+    ws = workspace(hx, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    combined, lse = hx.alltoall_combine_loopback(ins_o, ins_s, ws, hx.STATS_MAX_SUM, return_lse=True)
+    torch.cuda.synchronize()
+    assert ops.device_status() == 0
+    assert combined[0].shape == (w.tokens, w.heads_per_rank * w.head_dim) and lse[0].shape == (w.tokens, w.heads_per_rank)
+    want = oracle_combine(ins_o, ins_s, w.heads_per_rank, 1, ho.bf16_bits_to_f32)
+    check(combined, lse, want, "bf16")
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_combine_modes_dtypes_and_masked_heads(hx, ops, mode, dtype):
+    cp, tokens, heads, d = 4, 19, 3, 64
+    ws = workspace(hx, cp)
+    g = torch.Generator().manual_seed(mode * 2 + (dtype == torch.float16))
+    ins_o = [torch.randn(tokens, cp, heads * d, generator=g).to(dtype).cuda() for _ in range(cp)]
+    ins_s = []
+    for r in range(cp):
+        mx = torch.randn(tokens, cp, heads, generator=g) * 3
+        sm = 1 + torch.rand(tokens, cp, heads, generator=g) * 100
+        mx[torch.rand(tokens, cp, heads, generator=g) < 0.2] = float("-inf")  # fully masked shards
+        if r == 1:
+            mx[0] = float("-inf")  # a whole token masked on one rank
+        ins_s.append(torch.stack((mx, sm), -1).reshape(tokens, cp, 2 * heads).contiguous().cuda())
+    for t in ins_s:
+        t[1] = torch.where(torch.arange(2 * heads, device="cuda") % 2 == 0, float("-inf"), 1.0)  # every shard masked
+    ins_s[2][3, :, 0] = float("nan")   # NaN and +inf statistics count as masked
+    ins_s[3][4, :, 0] = float("inf")
+    combined, lse = hx.alltoall_combine_loopback(ins_o, ins_s, ws, mode, return_lse=True)
+    torch.cuda.synchronize()
+    assert ops.device_status() == 0
+    widen = ho.bf16_bits_to_f32 if dtype == torch.bfloat16 else ho.f16_bits_to_f32
+    want = oracle_combine(ins_o, ins_s, heads, mode, widen)
+    check(combined, lse, want, str(dtype))
+    for r in range(cp):
+        assert bool((combined[r][1] == 0).all()), "a head masked on every rank combines to zero"
+
+
+def test_combine_closed_forms(hx, ops):
+    # equal statistics -> arithmetic mean of the partial outputs; one dominant shard -> that shard
+    cp, tokens, heads, d = 8, 5, 2, 128
+    ws = workspace(hx, cp)
+    g = torch.Generator().manual_seed(3)
+    ins_o = [torch.randn(tokens, cp, heads * d, generator=g).to(torch.bfloat16).cuda() for _ in range(cp)]
+    equal = [torch.tensor([0.5, 7.0]).repeat(tokens, cp, heads).cuda() for _ in range(cp)]
+    combined = hx.alltoall_combine_loopback(ins_o, equal, ws, hx.STATS_MAX_SUM)
+    torch.cuda.synchronize()
+    for r in range(cp):
+        mean = torch.stack([ins_o[s][:, r, :].float() for s in range(cp)]).mean(0)
+        assert torch.allclose(combined[r].float(), mean, atol=ATOL, rtol=RTOL)
+    dominant = []
+    for s in range(cp):
+        lse = torch.full((tokens, cp, heads), 0.0 if s != 5 else 60.0)
+        dominant.append(torch.stack((lse, torch.zeros_like(lse)), -1).reshape(tokens, cp, 2 * heads).contiguous().cuda())
+    combined, lse = hx.alltoall_combine_loopback(ins_o, dominant, ws, hx.STATS_LSE, return_lse=True)
+    torch.cuda.synchronize()
+    assert ops.device_status() == 0
+    for r in range(cp):
+        assert torch.equal(combined[r], ins_o[5][:, r, :])      # weight 1 up to e^-60: bit-exact pass-through
+        assert torch.allclose(lse[r], torch.full_like(lse[r], 60.0))
+
+
+def test_combine_4d_inputs_and_plan_replay(hx, ops):
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS["c2"]
+    ws = workspace(hx, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    hp = w.heads_per_rank
+    o4 = [t.view(w.tokens, w.cp, hp, w.head_dim) for t in ins_o]
+    s4 = [t.view(w.tokens, w.cp, hp, 2) for t in ins_s]
+    plan = ops.CombinePlan(o4, s4, ws, ops.STATS_MAX_SUM, return_lse=False, channel_count=16)
+    want = oracle_combine(ins_o, ins_s, hp, 1, ho.bf16_bits_to_f32)
+    for _ in range(6):  # replays walk through the FIFO entries
+        combined = plan.run()
+    torch.cuda.synchronize()
+    assert ops.device_status() == 0
+    assert combined[0].shape == (w.tokens, hp, w.head_dim)
+    check(combined, None, want, "bf16")
+
+
+def test_combine_rejects_bad_shapes(hx, ops):
+    cp = 2
+    ws = workspace(hx, cp)
+    o = [torch.zeros(2, cp, 72, dtype=torch.bfloat16, device="cuda") for _ in range(cp)]   # 72 elements, 4 heads -> head_dim 18
+    s = [torch.zeros(2, cp, 8, device="cuda") for _ in range(cp)]
+    with pytest.raises(RuntimeError, match="head_dim"):
+        hx.alltoall_combine_loopback(o, s, ws)
+    with pytest.raises(RuntimeError, match="stats_mode"):
+        hx.alltoall_combine_loopback(o, s, ws, stats_mode=7)
+    big_o = [torch.zeros(1, 16, 8192, dtype=torch.bfloat16, device="cuda") for _ in range(16)]  # 16 x 16.5 KB > LDS
+    big_s = [torch.zeros(1, 16, 32, device="cuda") for _ in range(16)]
+    with pytest.raises(RuntimeError, match="LDS"):
+        hx.alltoall_combine_loopback(big_o, big_s, workspace(hx, 16))
