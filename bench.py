@@ -110,6 +110,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="c3")
     ap.add_argument("--channels", type=int, default=0, help="0 = automatic")
+    ap.add_argument("--combine", action="store_true", help="time the exchange fused with the LSE-weighted combine")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
@@ -136,7 +137,10 @@ def main() -> int:
     for r in range(w.cp):
         helix_a2a.init_workspace(ws, r, w.cp)
     ins_o, ins_s = make_inputs(w, "cuda")
-    plan = _ops.LoopbackPlan(ins_o, ins_s, ws, args.channels)
+    if args.combine:
+        plan = _ops.CombinePlan(ins_o, ins_s, ws, _ops.STATS_MAX_SUM, False, args.channels)
+    else:
+        plan = _ops.LoopbackPlan(ins_o, ins_s, ws, args.channels)
     channels = args.channels or _ops.auto_channel_count(w.cp, w.tokens)
 
     for _ in range(args.warmup):
@@ -158,7 +162,7 @@ def main() -> int:
     status = _ops.device_status()
     avg_kernel_ms = region_start.elapsed_time(region_end) / args.steps  # launch-to-launch, gaps included
     ms_per_step = wall * 1e3 / args.steps
-    bytes_per_call = w.exchange_bytes
+    bytes_per_call = w.combine_bytes if args.combine else w.exchange_bytes
 
     # distribution of single calls (event pair per call), outside the timed region
     n_dist = min(args.steps, 500)
@@ -173,7 +177,21 @@ def main() -> int:
     kernel_ms = sorted(s.elapsed_time(e) for s, e in zip(starts, ends))
 
     ok = status == 0
-    if not args.no_check:
+    if not args.no_check and args.combine:
+        import numpy as np
+
+        from helix_testing import torch_bits
+        combined = plan.run()
+        torch.cuda.synchronize()
+        recv_o = ho.exchange_closed_form([torch_bits(t) for t in ins_o])
+        recv_s = ho.exchange_closed_form([torch_bits(t) for t in ins_s])
+        for r in range(w.cp):
+            with np.errstate(all="ignore"):
+                want, _ = ho.combine_after_exchange(ho.bf16_bits_to_f32(recv_o[r]), recv_s[r].view(np.float32),
+                                                    w.heads_per_rank, 1)
+            got = combined[r].float().cpu().numpy()
+            ok &= bool((np.abs(got - want) <= 2e-2 + 2e-2 * np.abs(want)).all())
+    elif not args.no_check:
         outs_o, outs_s = plan.run()
         torch.cuda.synchronize()
         want_o, want_s = ho.exchange_single_copy(ins_o), ho.exchange_single_copy(ins_s)
@@ -203,12 +221,14 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "u8",
+        "dtype": "f32" if args.combine else "u8",
         "data": "synthetic",
-        "bit_exact": bool(ok),
+        "parity_ok": bool(ok),
+        "parity": "combined output within 2e-2 abs + 2e-2 rel of the oracle" if args.combine else "bit-exact against the oracle",
         "config": {
             "workload": f"{w.name}: Helix a2a loopback, cp={w.cp} logical ranks, T={w.tokens}, H={w.heads}, D={w.head_dim}, "
-                        f"partial_o bf16 [T,cp,H/cp,D] + softmax_stats fp32 [T,cp,H/cp,2], exchange only",
+                        f"partial_o bf16 [T,cp,H/cp,D] + softmax_stats fp32 [T,cp,H/cp,2], "
+                        + ("exchange fused with the LSE-weighted combine to bf16 [T,H/cp,D]" if args.combine else "exchange only"),
             "cp": w.cp, "T": w.tokens, "H": w.heads, "D": w.head_dim,
             "channels": channels,
             "algorithmic_bytes_per_call": bytes_per_call,
@@ -225,15 +245,15 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "helix_exchange_kernel",
+            "kernel": "helix_combine_kernel" if args.combine else "helix_exchange_kernel",
             "achieved": achieved,
             "peak": PEAK_HBM_GBPS,
             "unit": "GB/s",
             "frac": achieved / PEAK_HBM_GBPS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, channels)),
+            "traffic": None if args.combine else MEASURED_TRAFFIC_BYTES.get((w.name, channels)),
         },
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not args.combine:
         result["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(result))
     return 0 if ok else 1

@@ -392,9 +392,6 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, cons
   a.statsMode = stats_mode;
   a.dtype = dtype;
   a.headMagic = head_div_magic(static_cast<uint32_t>(a.headDim) * 2u / kPieceBytes);
-  const uint32_t lds = combine_lds_bytes(cp_size, plan.shape, heads);
-  if (lds > 159u * 1024u)
-    return fail(HELIX_A2A_ERR_CAPACITY, "combine needs %u bytes of LDS per workgroup (cp_size x message), more than a CU has", lds);
   const uint64_t outBytes = static_cast<uint64_t>(plan.entryCount) * a.field0Bytes;
   if (outBytes >= 2147483648ull) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "combined output exceeds 2 GiB");
   a.recvBytes0 = static_cast<uint32_t>(outBytes);
@@ -413,7 +410,20 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, cons
     a.entryBegin = begin;
     long end = static_cast<long>(begin) + plan.roundEntries;
     a.entryEnd = end > plan.entryCount ? plan.entryCount : static_cast<int>(end);
-    HELIX_HIP_TRY(launch_combine(a, static_cast<hipStream_t>(stream)));
+    // wavefronts per (receiver, channel): enough to cover a round's units once, and to fill the device
+    int msgs = stream_msg_count(a.entryBegin, a.entryEnd, 0, a.runChannels);
+    int perEntry = msgs_per_fifo_entry(plan.shape);
+    long runUnits = static_cast<long>(msgs < perEntry ? msgs : perEntry) * plan.shape.units;
+    long cover = (runUnits + kWaveLanes - 1) / kWaveLanes;
+    long fill = static_cast<long>(plan.cuCount) * 16 / (static_cast<long>(cp_size) * a.runChannels);
+    long parts = cover < fill ? cover : fill;
+    if (parts < 1) parts = 1;
+    if (parts > kMaxCombineParts) parts = kMaxCombineParts;
+    int p2 = 1;
+    while (p2 * 2 <= parts) p2 *= 2;
+    a.doSend = 1;
+    a.doRecv = 1;
+    HELIX_HIP_TRY(launch_combine(a, p2, static_cast<hipStream_t>(stream)));
   }
   return HELIX_A2A_OK;
 }

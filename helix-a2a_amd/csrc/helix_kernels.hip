@@ -78,6 +78,12 @@ struct SpinGuard {
   }
 };
 
+// Wait until every store this wavefront has issued is acknowledged. Used by a
+// sender before it moves `head`: FIFO lines are stored write-through (sc1), so
+// a `head` beyond a step tells any reader that the lines of that step are in
+// memory, all of them.
+__device__ __forceinline__ void wait_stores_acknowledged() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 __device__ __forceinline__ void raise_status(uint32_t* status, uint32_t bits, int lane) {
   if (lane == 0) atomicOr(status, bits);
 }
@@ -180,6 +186,7 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
         // open the FIFO entry of this run (csrc/helix_alltoall.cu:377-390)
         if (firstMsg > 0) {
           step += 1;
+          wait_stores_acknowledged();
           if (lane == 0) st_counter(&info[0], step);
         }
         SpinGuard guard(a.spinLimitTicks);
@@ -206,6 +213,7 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
       }
     }
   }
+  wait_stores_acknowledged();
   if (lane == 0) st_counter(&info[0], step + 1);  // close the last entry (csrc/helix_alltoall.cu:409-412)
 }
 
@@ -228,6 +236,10 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
   st.stride1 = a.recvStride1;
 
   int64_t step = info[1];
+  // The sender's head is the acquire token of a whole run: once it is beyond
+  // `step`, every line of that step is in memory (the sender waits for its
+  // stores before it moves head) and the run can be read in one pass.
+  int64_t head = ld_counter(&senderInfo[0]);
   const int flagLane = lane | 7;
 
   for (int firstMsg = 0; firstMsg < st.msgs; firstMsg += st.msgsPerEntry) {
@@ -241,7 +253,9 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
         st_counter(&info[1], step);
         st_counter(&senderInfo[1], step);
       }
+      if (head <= step) head = ld_counter(&senderInfo[0]);
     }
+    bool runClosed = head > step;
     const uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
     const uint32_t stepLo = static_cast<uint32_t>(step);
     const uint32_t stepHi = static_cast<uint32_t>(static_cast<uint64_t>(step) >> 32);
@@ -251,32 +265,61 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
       for (int i = 0; i < kUnitsInFlight; ++i) pending[i] = (U0 + i * kWaveLanes + lane) < runUnits;
       SpinGuard guard(a.spinLimitTicks);
       for (;;) {
+        bool landed[kUnitsInFlight];
+        if (runClosed) {
+#pragma unroll
+          for (int i = 0; i < kUnitsInFlight; ++i) landed[i] = pending[i];
+        } else {
+          // The sender may still be writing. Acquire line by line: first the flag
+          // words (upper half of each line's last unit, loaded by the eight flag
+          // lanes only), then -- with offsets that depend on what those loads
+          // returned -- the units of the lines whose flag carries the step. A unit
+          // is never read before its line's flag was seen, whatever the
+          // granularity at which the memory system serves a 128-byte line.
+#pragma unroll
+          for (int i = 0; i < kUnitsInFlight; ++i) {
+            uint32_t U = U0 + i * kWaveLanes + lane;
+            bool isFlagLane = (U & 7u) == 7u;
+            uint32_t off = (pending[i] && isFlagLane) ? entryOffset + U * kUnitBytes + kPieceBytes : kOutOfRange;
+            u32x2 f = __builtin_amdgcn_raw_buffer_load_b64(st.fifo, off, 0, kAux);
+            bool ok = !pending[i] || !isFlagLane || (f.x == stepLo && f.y == stepHi);
+            unsigned long long okMask = __ballot(ok);
+            landed[i] = pending[i] && ((okMask >> flagLane) & 1ull) != 0ull;
+          }
+        }
         u32x4 v[kUnitsInFlight];
 #pragma unroll
         for (int i = 0; i < kUnitsInFlight; ++i) {
           uint32_t U = U0 + i * kWaveLanes + lane;
-          uint32_t off = pending[i] ? entryOffset + U * kUnitBytes : kOutOfRange;
+          uint32_t off = landed[i] ? entryOffset + U * kUnitBytes : kOutOfRange;
           v[i] = __builtin_amdgcn_raw_buffer_load_b128(st.fifo, off, 0, kAux);
         }
+        // every unit that is consumed carries its line's flag in the very load that brought it
         bool anyPending = false;
-        bool landed[kUnitsInFlight];
-        bool needField1 = false;
+        bool flagsAgree = true;
 #pragma unroll
         for (int i = 0; i < kUnitsInFlight; ++i) {
           uint32_t U = U0 + i * kWaveLanes + lane;
           bool isFlagLane = (U & 7u) == 7u;
-          bool ok = !pending[i] || !isFlagLane || (v[i].z == stepLo && v[i].w == stepHi);
+          bool ok = !landed[i] || !isFlagLane || (v[i].z == stepLo && v[i].w == stepHi);
           unsigned long long okMask = __ballot(ok);
-          bool lineOk = (okMask >> flagLane) & 1ull;
-          landed[i] = pending[i] && lineOk;
+          bool lineOk = ((okMask >> flagLane) & 1ull) != 0ull;
+          flagsAgree &= !landed[i] || lineOk;
+          landed[i] = landed[i] && lineOk;
+          pending[i] = pending[i] && !landed[i];
+          anyPending |= pending[i];
+        }
+        if (__ballot(!flagsAgree) != 0ull) runClosed = false;  // not what the token promised: go line by line
+        bool needField1 = false;
+#pragma unroll
+        for (int i = 0; i < kUnitsInFlight; ++i) {
+          uint32_t U = U0 + i * kWaveLanes + lane;
           UnitOffsets o = unit_offsets(st, firstMsg, U, landed[i]);
           u32x2 wa = {v[i].x, v[i].y};
           u32x2 wb = {v[i].z, v[i].w};
           __builtin_amdgcn_raw_buffer_store_b64(wa, st.field0, o.a0, 0, kAuxNone);
           __builtin_amdgcn_raw_buffer_store_b64(wb, st.field0, o.b0, 0, kAuxNone);
           needField1 |= (o.a1 != kOutOfRange) | (o.b1 != kOutOfRange);
-          pending[i] = pending[i] && !lineOk;
-          anyPending |= pending[i];
         }
         if (__ballot(needField1) != 0ull) {
 #pragma unroll
@@ -364,178 +407,306 @@ __device__ __forceinline__ uint32_t narrow1<1>(float v) {
   return static_cast<uint32_t>(__half_as_ushort(__float2half_rn(v)));
 }
 
-// Receive half of the fused form: the cpSize wavefronts of a workgroup each
-// poll one sender's FIFO for the same (receiver, channel), park the payload
-// pieces in LDS, and the workgroup then reduces over the senders:
+// Receive half of the fused form. A wavefront serves one (receiver, channel)
+// and all cpSize senders at once: lane L owns run unit U (the same unit of
+// the same message in every sender's FIFO, since all streams of a channel
+// share one layout), loads that unit from each sender's FIFO, and reduces
+// over the senders in registers:
 //   out[e, h, :] = sum_s w[s, h] * partial_o_s[e, h, :],  w = softmax_s(lse[s, h])
-// (patches/dcp_alltoall_helix.py:142-207). LDS: [cp][np] pieces, then [cp][heads] weights.
-template <int kDtype>
-__device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r, int s, int ch, int lane,
-                                                     uint8_t* lds, int* failed) {
-  Stream st;
-  setup_stream(st, a, s, ch);
-  if (st.msgs == 0) return;  // uniform over the workgroup: same channel
-  uint8_t* senderRow = a.workspace + static_cast<uint64_t>(s) * a.rowStrideBytes;
-  uint8_t* receiverRow = a.workspace + static_cast<uint64_t>(r) * a.rowStrideBytes;
-  int64_t* senderInfo = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(a.cpSize, a.maxChannels, r, ch));
-  int64_t* info = reinterpret_cast<int64_t*>(receiverRow + receiver_info_offset(a.cpSize, a.maxChannels, s, ch));
-  st.fifo = make_rsrc(receiverRow + fifo_offset(s, ch, a.maxChannels), kFifoBytes);
-  __amdgpu_buffer_rsrc_t outRsrc = make_rsrc(a.rank[r].recv0, a.recvBytes0);
-  float* lseOut = reinterpret_cast<float*>(a.rank[r].recv1);
+// (patches/dcp_alltoall_helix.py:142-207). The statistics of head h live in
+// piece np0 + h of each message. Every distinct statistics line the lanes of
+// a wavefront need is fetched once per wavefront, by lanes 0..7 in the
+// pattern of a payload line (lane u takes unit u, so the line is validated by
+// its own flag unit in the same load), and handed to the lanes that need it
+// with lane shuffles. The softmax runs online over groups of eight senders,
+// so nothing but two accumulators survives a group. The `parts` wavefronts of
+// a workgroup split the units of a run between them. No LDS, one barrier.
+// The kernel is bounded by instruction issue rather than by memory: exp and
+// ln use the hardware's base-2 units.
+struct CombineCtx {
+  __amdgpu_buffer_rsrc_t fifos;  // the whole FIFO region of the receiver's row
+  uint32_t channelBase;          // byte offset of sender 0's FIFO of this channel
+  uint32_t senderStride;         // bytes between the FIFOs of consecutive senders
+  uint32_t stepLo, stepHi;       // lane q: step counter of sender q's stream
+};
 
-  u32x2* pieces = reinterpret_cast<u32x2*>(lds);                                    // [cp][np]
-  float* weights = reinterpret_cast<float*>(lds + static_cast<size_t>(a.cpSize) * st.np * kPieceBytes);  // [cp][heads]
-  u32x2* myPieces = pieces + static_cast<size_t>(s) * st.np;
+__device__ __forceinline__ uint32_t lane_value(uint32_t v, int q) {
+  return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), q));
+}
+__device__ __forceinline__ uint32_t shuffle_from(uint32_t v, int srcLane) {
+  return static_cast<uint32_t>(__shfl(static_cast<int>(v), srcLane, kWaveLanes));
+}
 
-  int64_t step = info[1];
-  const int flagLane = lane | 7;
-  const int tid = static_cast<int>(threadIdx.x);
-  const int threads = static_cast<int>(blockDim.x);
+// byte offset of sender q's open FIFO entry inside the receiver's FIFO region
+__device__ __forceinline__ uint32_t entry_base(const CombineCtx& cx, int q, uint32_t stepLo) {
+  return cx.channelBase + static_cast<uint32_t>(q) * cx.senderStride + (stepLo & (kFifoDepth - 1)) * kFifoEntryBytes;
+}
 
-  for (int k = 0; k < st.msgs; ++k) {
-    const int posInRun = k % st.msgsPerEntry;
-    if (k > 0 && posInRun == 0) {
-      step += 1;
-      if (lane == 0) {
-        st_counter(&info[1], step);
-        st_counter(&senderInfo[1], step);
-      }
-    }
-    const uint32_t msgOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes +
-                               static_cast<uint32_t>(posInRun) * st.lines * kLineBytes;
-    const uint32_t stepLo = static_cast<uint32_t>(step);
-    const uint32_t stepHi = static_cast<uint32_t>(static_cast<uint64_t>(step) >> 32);
-    bool timedOut = false;
-    for (uint32_t U0 = 0; U0 < st.unitsPerMsg && !timedOut; U0 += kUnitsInFlight * kWaveLanes) {
-      bool pending[kUnitsInFlight];
+// exp and ln on the hardware's base-2 units (v_exp_f32 / v_log_f32, about 1 ulp):
+// the combine is bounded by instruction issue, and its result is rounded to
+// 8 mantissa bits anyway. exp(-inf) = 0, ln(0) = -inf, ln(x < 0) = NaN hold.
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+__device__ __forceinline__ float fast_log(float x) { return __builtin_amdgcn_logf(x) * 0.6931471805599453f; }
+
+// Running softmax-weighted sum of one 8-byte piece (4 elements) over the senders.
+struct OnlineSum {
+  float m, total;
+  float acc[4];
+  __device__ __forceinline__ void init() {
+    m = -INFINITY;
+    total = 0.0f;
+    acc[0] = acc[1] = acc[2] = acc[3] = 0.0f;
+  }
+  // raise the running maximum to cover `candidate`
+  __device__ __forceinline__ void rescale(float candidate) {
+    float mNew = fmaxf(m, candidate);
+    float scale = (mNew == -INFINITY) ? 1.0f : fast_exp(m - mNew);  // m == -inf: nothing accumulated yet, scale is 0
+    m = mNew;
+    total *= scale;
 #pragma unroll
-      for (int i = 0; i < kUnitsInFlight; ++i) pending[i] = (U0 + i * kWaveLanes + lane) < st.unitsPerMsg;
+    for (int c = 0; c < 4; ++c) acc[c] *= scale;
+  }
+  __device__ __forceinline__ float weight(float lse) const { return (m == -INFINITY) ? 0.0f : fast_exp(lse - m); }
+  __device__ __forceinline__ void add(float e, const float (&f)[4]) {
+    total += e;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] += e * f[c];
+  }
+  __device__ __forceinline__ float lse_value() const { return fast_log(total) + (m == -INFINITY ? 0.0f : m); }
+  __device__ __forceinline__ float inv_total() const { return 1.0f / fmaxf(total, 1e-10f); }
+};
+
+// log-sum-exp of one {stats[2h], stats[2h+1]} pair; NaN and +-inf count as "no contribution"
+__device__ __forceinline__ float lse_of_stats(uint32_t s0, uint32_t s1, int statsMode) {
+  float x = __uint_as_float(s0);
+  if (statsMode == 1) x = x + fast_log(__uint_as_float(s1));  // running max + ln(running sum)
+  return (isnan(x) || isinf(x)) ? -INFINITY : x;
+}
+
+template <int kDtype>
+__device__ __forceinline__ u32x2 narrow_piece(const OnlineSum& o) {
+  const float inv = o.inv_total();
+  u32x2 r = {narrow1<kDtype>(o.acc[0] * inv) | (narrow1<kDtype>(o.acc[1] * inv) << 16),
+             narrow1<kDtype>(o.acc[2] * inv) | (narrow1<kDtype>(o.acc[3] * inv) << 16)};
+  return r;
+}
+
+template <int kDtype>
+__device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r, int ch, int part, int parts,
+                                                     int lane) {
+  constexpr int kGroup = 8;  // senders whose loads are in flight together
+  Stream st;
+  setup_stream(st, a, 0, ch);
+  if (st.msgs == 0) return;  // uniform over the workgroup: same channel
+  uint8_t* receiverRow = a.workspace + static_cast<uint64_t>(r) * a.rowStrideBytes;
+  CombineCtx cx;
+  cx.fifos = make_rsrc(receiverRow, static_cast<uint32_t>(fifo_region_bytes(a.cpSize, a.maxChannels)));
+  cx.channelBase = static_cast<uint32_t>(fifo_offset(0, ch, a.maxChannels));
+  cx.senderStride = static_cast<uint32_t>(fifo_offset(1, 0, a.maxChannels));
+  __amdgpu_buffer_rsrc_t outRsrc = make_rsrc(a.rank[r].recv0, a.recvBytes0);
+  __amdgpu_buffer_rsrc_t lseRsrc = make_rsrc(a.rank[r].recv1, a.rank[r].recv1 ? a.recvBytes1 : 0u);
+  const uint32_t piecesPerHead = static_cast<uint32_t>(a.headDim) * 2u / kPieceBytes;
+  const int flagLane = lane | 7;
+
+  // lane q owns the counters of sender q's stream
+  int64_t myStep = 0;
+  int64_t* myInfo = nullptr;
+  int64_t* mySenderInfo = nullptr;
+  if (lane < a.cpSize) {
+    uint8_t* senderRow = a.workspace + static_cast<uint64_t>(lane) * a.rowStrideBytes;
+    myInfo = reinterpret_cast<int64_t*>(receiverRow + receiver_info_offset(a.cpSize, a.maxChannels, lane, ch));
+    mySenderInfo = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(a.cpSize, a.maxChannels, r, ch));
+    myStep = myInfo[1];
+  }
+  __syncthreads();  // every part has read the counters before part 0 moves them
+  if (part == 0 && lane < a.cpSize) {
+    // rounds never put more than the four entries in flight, so the entries can
+    // be handed back up front; nothing reads these counters before the launch ends
+    const MsgShape sh = make_msg_shape(a.field0Bytes, a.field1Bytes);
+    int64_t done = myStep + entries_for_msgs(st.msgs, sh);
+    st_counter(&myInfo[1], done);
+    st_counter(&mySenderInfo[1], done);
+  }
+
+  for (int firstMsg = 0; firstMsg < st.msgs; firstMsg += st.msgsPerEntry, myStep += 1) {
+    const int runMsgs = min(st.msgsPerEntry, st.msgs - firstMsg);
+    const uint32_t runUnits = static_cast<uint32_t>(runMsgs) * st.unitsPerMsg;
+    cx.stepLo = static_cast<uint32_t>(myStep);
+    cx.stepHi = static_cast<uint32_t>(static_cast<uint64_t>(myStep) >> 32);
+    {
+      // Acquire the run from every sender: a head beyond the step says that all
+      // lines of the step are in memory (the sender waits for its stores before
+      // it moves head). Every unit needs all cpSize senders anyway.
       SpinGuard guard(a.spinLimitTicks);
       for (;;) {
-        u32x4 v[kUnitsInFlight];
-#pragma unroll
-        for (int i = 0; i < kUnitsInFlight; ++i) {
-          uint32_t U = U0 + i * kWaveLanes + lane;
-          uint32_t off = pending[i] ? msgOffset + U * kUnitBytes : kOutOfRange;
-          v[i] = __builtin_amdgcn_raw_buffer_load_b128(st.fifo, off, 0, kAuxSc1);
+        const bool closed = lane >= a.cpSize || ld_counter(&mySenderInfo[0]) > myStep;
+        if (__ballot(!closed) == 0ull) break;
+        if (guard.expired()) {
+          raise_status(a.status, kStatusRecvTimeout, lane);
+          return;
         }
-        bool anyPending = false;
+        __builtin_amdgcn_s_sleep(8);
+      }
+      asm volatile("" ::: "memory");
+    }
+    for (uint32_t U0 = static_cast<uint32_t>(part) * kWaveLanes; U0 < runUnits;
+         U0 += static_cast<uint32_t>(parts) * kWaveLanes) {
+      const uint32_t U = U0 + lane;
+      const RunUnit d = decode_run_unit(U, st.lines, st.magic);
+      const bool live = U < runUnits;
+      const bool dataA = live && d.piece0 < st.np0;
+      const bool dataB = live && !d.flag && d.piece0 + 1 < st.np0;
+      if (__ballot(dataA) == 0ull) continue;  // statistics, padding: nothing to reduce here
+      const uint32_t hA = head_of_piece(d.piece0, a.headMagic);
+      const uint32_t hB = dataB ? head_of_piece(d.piece0 + 1, a.headMagic) : hA;
+      const uint32_t entry = static_cast<uint32_t>(a.entryBegin + ch) + (firstMsg + d.msg) * a.runChannels;
+      // where the statistics of heads hA / hB sit: run line and word inside it
+      const uint32_t psA = st.np0 + hA, psB = st.np0 + hB;
+      const uint32_t lineA = d.msg * st.lines + psA / kPiecesPerLine, wordA = psA % kPiecesPerLine;
+      const uint32_t lineB = d.msg * st.lines + psB / kPiecesPerLine, wordB = psB % kPiecesPerLine;
+      // piece B shares the weights of piece A unless it starts the next head
+      const bool ownB = dataB && hB != hA;
+      const bool anyOwnB = __ballot(ownB) != 0ull;
+
+      OnlineSum sumA, sumB;
+      sumA.init();
+      sumB.init();
+
+      for (int g = 0; g < a.cpSize; g += kGroup) {
+        u32x4 v[kGroup];
+        float lseA[kGroup], lseB[kGroup];
+        SpinGuard guard(a.spinLimitTicks);
+        for (;;) {
+          // payload unit of every sender of the group
 #pragma unroll
-        for (int i = 0; i < kUnitsInFlight; ++i) {
-          uint32_t U = U0 + i * kWaveLanes + lane;
-          bool isFlagLane = (U & 7u) == 7u;
-          bool ok = !pending[i] || !isFlagLane || (v[i].z == stepLo && v[i].w == stepHi);
-          unsigned long long okMask = __ballot(ok);
-          bool lineOk = (okMask >> flagLane) & 1ull;
-          if (pending[i] && lineOk) {
-            uint32_t pa = static_cast<uint32_t>(unit_first_piece(static_cast<int>(U)));
-            if (pa < st.np) {
-              u32x2 wa = {v[i].x, v[i].y};
-              myPieces[pa] = wa;
-            }
-            if (!isFlagLane && pa + 1 < st.np) {
-              u32x2 wb = {v[i].z, v[i].w};
-              myPieces[pa + 1] = wb;
+          for (int j = 0; j < kGroup; ++j) {
+            const int q = g + j;
+            if (q < a.cpSize) {
+              const uint32_t base = entry_base(cx, q, lane_value(cx.stepLo, q));
+              v[j] = __builtin_amdgcn_raw_buffer_load_b128(cx.fifos, live ? base + U * kUnitBytes : kOutOfRange, 0, kAuxSc1);
             }
           }
-          pending[i] = pending[i] && !lineOk;
-          anyPending |= pending[i];
-        }
-        if (__ballot(anyPending) == 0ull) break;
-        if (guard.expired()) {
-          timedOut = true;
-          break;
-        }
-        __builtin_amdgcn_s_sleep(1);
-        asm volatile("" ::: "memory");
-      }
-    }
-    if (timedOut) {
-      raise_status(a.status, kStatusRecvTimeout, lane);
-      if (lane == 0) atomicOr(failed, 1);
-    }
-    __syncthreads();
-    if (*failed) return;  // every wavefront of the workgroup sees the same value here
-
-    // weights of every (sender, head): softmax over the senders of the log-sum-exp
-    const int entry = a.entryBegin + ch + k * a.runChannels;
-    for (int h = tid; h < a.heads; h += threads) {
-      float lse[kMaxCpSize];
-      float m = -INFINITY;
+          // Statistics: every distinct line some lane needs is fetched once per
+          // wavefront, by lanes 0..7 in the pattern of a payload line (lane u takes
+          // unit u, so the line is validated by its own flag unit in the same
+          // load), and handed to the lanes that need it with lane shuffles.
+          bool ok = true;
+          bool pendA = dataA, pendB = ownB;
+          for (;;) {
+            const unsigned long long need = __ballot(pendA || pendB);
+            if (need == 0ull) break;
+            const int leader = __ffsll(static_cast<long long>(need)) - 1;
+            const uint32_t line = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(pendA ? lineA : lineB), leader));
+            const bool takeA = pendA && lineA == line, takeB = pendB && lineB == line;
+            const uint32_t unitOff = line * kLineBytes + static_cast<uint32_t>(lane) * kUnitBytes;
 #pragma unroll
-      for (int q = 0; q < kMaxCpSize; ++q) {
-        if (q < a.cpSize) {
-          u32x2 st2 = pieces[static_cast<size_t>(q) * st.np + st.np0 + h];  // {stats[2h], stats[2h+1]}
-          float x = __uint_as_float(st2.x);
-          if (a.statsMode == 1) x = x + logf(__uint_as_float(st2.y));   // running max + ln(running sum)
-          if (isnan(x) || isinf(x)) x = -INFINITY;
-          lse[q] = x;
-          m = fmaxf(m, x);
+            for (int j = 0; j < kGroup; ++j) {
+              const int q = g + j;
+              if (q < a.cpSize) {
+                const uint32_t sLo = lane_value(cx.stepLo, q), sHi = lane_value(cx.stepHi, q);
+                const uint32_t base = entry_base(cx, q, sLo);
+                const u32x4 sv = __builtin_amdgcn_raw_buffer_load_b128(cx.fifos, lane < 8 ? base + unitOff : kOutOfRange, 0, kAuxSc1);
+                const unsigned long long landed = __ballot(lane != 7 || (sv.z == sLo && sv.w == sHi));
+                ok &= ((landed >> 7) & 1ull) != 0ull;
+                // every lane takes part in every shuffle (a lane can only be read while it is active)
+                const int srcA = static_cast<int>(wordA >> 1);
+                const uint32_t ax = shuffle_from(sv.x, srcA), ay = shuffle_from(sv.y, srcA);
+                const uint32_t az = shuffle_from(sv.z, srcA), aw = shuffle_from(sv.w, srcA);
+                const float la = lse_of_stats((wordA & 1u) ? az : ax, (wordA & 1u) ? aw : ay, a.statsMode);
+                if (takeA) lseA[j] = la;
+                if (anyOwnB) {
+                  const int srcB = static_cast<int>(wordB >> 1);
+                  const uint32_t bx = shuffle_from(sv.x, srcB), by = shuffle_from(sv.y, srcB);
+                  const uint32_t bz = shuffle_from(sv.z, srcB), bw = shuffle_from(sv.w, srcB);
+                  const float lb = lse_of_stats((wordB & 1u) ? bz : bx, (wordB & 1u) ? bw : by, a.statsMode);
+                  if (takeB) lseB[j] = lb;
+                }
+              }
+            }
+            pendA = pendA && !takeA;
+            pendB = pendB && !takeB;
+          }
+          // payload lines: flag unit of each line, shared through a ballot
+#pragma unroll
+          for (int j = 0; j < kGroup; ++j) {
+            const int q = g + j;
+            if (q < a.cpSize) {
+              const uint32_t sLo = lane_value(cx.stepLo, q), sHi = lane_value(cx.stepHi, q);
+              const unsigned long long landed = __ballot(!(live && d.flag) || (v[j].z == sLo && v[j].w == sHi));
+              ok &= ((landed >> flagLane) & 1ull) != 0ull;
+            }
+          }
+          if (__ballot(!ok) == 0ull) break;
+          if (guard.expired()) {
+            raise_status(a.status, kStatusRecvTimeout, lane);
+            return;
+          }
+          __builtin_amdgcn_s_sleep(16);
+          asm volatile("" ::: "memory");
+        }
+        float gmaxA = -INFINITY, gmaxB = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < kGroup; ++j) {
+          if (g + j < a.cpSize) {
+            if (!dataA) lseA[j] = -INFINITY;
+            if (!ownB) lseB[j] = lseA[j];
+            gmaxA = fmaxf(gmaxA, lseA[j]);
+            gmaxB = fmaxf(gmaxB, lseB[j]);
+          }
+        }
+        sumA.rescale(gmaxA);
+        sumB.rescale(gmaxB);  // equals gmaxA for every lane whose second piece shares the head
+#pragma unroll
+        for (int j = 0; j < kGroup; ++j) {
+          if (g + j < a.cpSize) {
+            float f[4];
+            u32x2 pa = {v[j].x, v[j].y};
+            u32x2 pb = {v[j].z, v[j].w};
+            const float ea = sumA.weight(lseA[j]);
+            widen4<kDtype>(pa, f);
+            sumA.add(ea, f);
+            const float eb = anyOwnB ? sumB.weight(lseB[j]) : ea;
+            widen4<kDtype>(pb, f);
+            sumB.add(eb, f);
+          }
         }
       }
-      if (m == -INFINITY) m = 0.0f;
-      float total = 0.0f;
-#pragma unroll
-      for (int q = 0; q < kMaxCpSize; ++q) {
-        if (q < a.cpSize) {
-          float w = expf(lse[q] - m);
-          if (isnan(w)) w = 0.0f;
-          lse[q] = w;
-          total += w;
-        }
-      }
-      float inv = 1.0f / fmaxf(total, 1e-10f);
-#pragma unroll
-      for (int q = 0; q < kMaxCpSize; ++q) {
-        if (q < a.cpSize) weights[q * a.heads + h] = lse[q] * inv;
-      }
-      if (lseOut != nullptr) lseOut[static_cast<size_t>(entry) * a.heads + h] = logf(total) + m;
+      // the lane that holds the first piece of a head reports that head's log-sum-exp
+      const bool reportA = dataA && d.piece0 == hA * piecesPerHead;
+      const bool reportB = dataB && d.piece0 + 1 == hB * piecesPerHead;
+      __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(sumA.lse_value()), lseRsrc,
+                                            reportA ? (entry * a.heads + hA) * 4u : kOutOfRange, 0, kAuxNone);
+      __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(sumB.lse_value()), lseRsrc,
+                                            reportB ? (entry * a.heads + hB) * 4u : kOutOfRange, 0, kAuxNone);
+      const uint32_t rowByte = entry * (st.np0 * kPieceBytes);
+      __builtin_amdgcn_raw_buffer_store_b64(narrow_piece<kDtype>(sumA), outRsrc,
+                                            dataA ? rowByte + d.piece0 * kPieceBytes : kOutOfRange, 0, kAuxNone);
+      __builtin_amdgcn_raw_buffer_store_b64(narrow_piece<kDtype>(sumB), outRsrc,
+                                            dataB ? rowByte + (d.piece0 + 1) * kPieceBytes : kOutOfRange, 0, kAuxNone);
     }
-    __syncthreads();
-
-    // weighted sum over the senders, 4 elements (one piece) per thread and step
-    for (uint32_t j = static_cast<uint32_t>(tid); j < st.np0; j += static_cast<uint32_t>(threads)) {
-      uint32_t h = head_of_piece(j, a.headMagic);
-      float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-      for (int q = 0; q < a.cpSize; ++q) {
-        float f[4];
-        widen4<kDtype>(pieces[static_cast<size_t>(q) * st.np + j], f);
-        float w = weights[q * a.heads + h];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) acc[c] += w * f[c];
-      }
-      u32x2 o = {narrow1<kDtype>(acc[0]) | (narrow1<kDtype>(acc[1]) << 16),
-                 narrow1<kDtype>(acc[2]) | (narrow1<kDtype>(acc[3]) << 16)};
-      uint32_t off = static_cast<uint32_t>(entry) * (st.np0 * kPieceBytes) + j * kPieceBytes;
-      __builtin_amdgcn_raw_buffer_store_b64(o, outRsrc, off, 0, kAuxNone);
-    }
-    __syncthreads();  // LDS is reused by the next message
-  }
-  if (lane == 0) {
-    st_counter(&info[1], step + 1);
-    st_counter(&senderInfo[1], step + 1);
   }
 }
 
-// Workgroups of cpSize wavefronts. The first rankCount*runChannels workgroups
-// send (workgroup = (sender, channel), wavefront = receiver), the rest receive
-// and combine (workgroup = (receiver, channel), wavefront = sender).
+// Workgroups of `parts` wavefronts (blockDim.x / 64). The first
+// ceil(senderStreams / parts) workgroups send, one stream per wavefront; the
+// rest receive and combine, one workgroup per (receiver, channel).
 template <int kDtype>
-__global__ __launch_bounds__(kMaxCpSize * kWaveLanes) void helix_combine_kernel(KernelArgs a) {
-  extern __shared__ __align__(16) uint8_t dynamicLds[];
-  __shared__ int failed;
+__global__ __launch_bounds__(kMaxCombineParts * kWaveLanes) void helix_combine_kernel(KernelArgs a) {
+  const int parts = static_cast<int>(blockDim.x) / kWaveLanes;
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWaveLanes);
   const int lane = static_cast<int>(threadIdx.x) % kWaveLanes;
-  const int sendBlocks = a.rankCount * a.runChannels;
+  const int senderStreams = a.doSend ? a.rankCount * a.runChannels * a.cpSize : 0;
+  const int sendBlocks = (senderStreams + parts - 1) / parts;
   int b = static_cast<int>(blockIdx.x);
   if (b < sendBlocks) {
-    run_sender<kAuxSc1>(a, a.rankBegin + b / a.runChannels, wave, b % a.runChannels, lane);
+    const int w = b * parts + wave;
+    if (w >= senderStreams) return;
+    const int t = w / a.cpSize;
+    run_sender<kAuxSc1>(a, a.rankBegin + t / a.runChannels, w % a.cpSize, t % a.runChannels, lane);
     return;
   }
   b -= sendBlocks;
-  if (threadIdx.x == 0) failed = 0;
-  __syncthreads();
-  run_combine_receiver<kDtype>(a, a.rankBegin + b / a.runChannels, wave, b % a.runChannels, lane, dynamicLds, &failed);
+  run_combine_receiver<kDtype>(a, a.rankBegin + b / a.runChannels, b % a.runChannels, wave, parts, lane);
 }
 
 // FIFO region <- 0xFF bytes, info regions <- 0 (csrc/helix_alltoall.cu:637-643).
@@ -559,26 +730,17 @@ hipError_t launch_exchange(const KernelArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_combine(const KernelArgs& a, hipStream_t stream) {
-  int blocks = 2 * a.rankCount * a.runChannels;
-  if (blocks <= 0) return hipSuccess;
-  const MsgShape sh = make_msg_shape(a.field0Bytes, a.field1Bytes);
-  uint32_t lds = combine_lds_bytes(a.cpSize, sh, a.heads);
-  dim3 block(static_cast<unsigned>(a.cpSize * kWaveLanes));
+hipError_t launch_combine(const KernelArgs& a, int parts, hipStream_t stream) {
+  const int senderStreams = a.doSend ? a.rankCount * a.runChannels * a.cpSize : 0;
+  if (a.rankCount * a.runChannels <= 0) return hipSuccess;
+  if (parts < 1) parts = 1;
+  if (parts > kMaxCombineParts) parts = kMaxCombineParts;
+  const int blocks = (senderStreams + parts - 1) / parts + a.rankCount * a.runChannels;
+  dim3 block(static_cast<unsigned>(parts * kWaveLanes));
   if (a.dtype == 1) {
-    if (lds > 64u * 1024u) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&helix_combine_kernel<1>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-      if (e != hipSuccess) return e;
-    }
-    hipLaunchKernelGGL(helix_combine_kernel<1>, dim3(blocks), block, lds, stream, a);
+    hipLaunchKernelGGL(helix_combine_kernel<1>, dim3(blocks), block, 0, stream, a);
   } else {
-    if (lds > 64u * 1024u) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&helix_combine_kernel<0>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-      if (e != hipSuccess) return e;
-    }
-    hipLaunchKernelGGL(helix_combine_kernel<0>, dim3(blocks), block, lds, stream, a);
+    hipLaunchKernelGGL(helix_combine_kernel<0>, dim3(blocks), block, 0, stream, a);
   }
   return hipGetLastError();
 }

@@ -52,12 +52,10 @@ constexpr int kBlockThreads = kWavesPerBlock * kWaveLanes;
 inline int waves_per_direction(const KernelArgs& a) { return a.rankCount * a.runChannels * a.cpSize; }
 
 hipError_t launch_exchange(const KernelArgs& a, hipStream_t stream);
-// exchange fused with the LSE-weighted combine, all ranks of the launch; workgroups of cpSize wavefronts
-hipError_t launch_combine(const KernelArgs& a, hipStream_t stream);
-// bytes of LDS a combine workgroup needs
-inline uint32_t combine_lds_bytes(int cpSize, const MsgShape& sh, int heads) {
-  return static_cast<uint32_t>(cpSize) * sh.np * kPieceBytes + static_cast<uint32_t>(cpSize) * heads * 4u;
-}
+// exchange fused with the LSE-weighted combine, all ranks of the launch; `parts` wavefronts share
+// the units of one (receiver, channel)
+constexpr int kMaxCombineParts = 8;
+hipError_t launch_combine(const KernelArgs& a, int parts, hipStream_t stream);
 hipError_t launch_init_row(uint8_t* row, uint64_t fifoBytes, uint64_t infoBytes, hipStream_t stream);
 
 }  // namespace helix

@@ -503,3 +503,28 @@ def test_traffic_beyond_fifo_capacity(hx, ops, single_round):
         ops.set_single_round(False)
     assert_clean(ops)
     check_against_oracle(ins_o, ins_s, outs_o, outs_s)
+
+
+@pytest.mark.parametrize("channels", [8, 16])
+def test_receivers_overlapping_their_senders(hx, ops, channels):
+    # With few channels every wavefront of the launch is resident at once and receivers poll FIFO
+    # lines while their senders are still writing them. A receiver that consumed a line on the
+    # strength of a flag it had read in the same pass as the payload could see a half-written line.
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS["c3"]
+    ws = get_workspace(hx, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    want_o = expected_on_device(ins_o).view(torch.int16)
+    want_s = expected_on_device(ins_s).view(torch.int32)
+    plan = ops.LoopbackPlan(ins_o, ins_s, ws, channels)
+    bad = torch.zeros((), dtype=torch.int64, device="cuda")
+    for _ in range(150):
+        for t in plan.out_o:
+            t.zero_()
+        outs_o, outs_s = plan.run()
+        for r in range(w.cp):
+            bad += (outs_o[r].view(torch.int16) != want_o[r]).sum() + (outs_s[r].view(torch.int32) != want_s[r]).sum()
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    assert int(bad.item()) == 0
