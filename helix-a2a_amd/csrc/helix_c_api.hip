@@ -94,17 +94,17 @@ int check_cp_size(int cpSize) {
   return HELIX_A2A_OK;
 }
 
-// One wavefront per (sender, receiver, channel) and direction; aim for one
-// resident wavefront slot per sender stream on a device that holds
-// 32 wavefronts per CU, and never more channels than entries.
+// One wavefront per (sender, receiver, channel) and direction. A wavefront
+// walks its stream's messages one chunk after the other, so the exchange gets
+// faster with every channel that still has an entry to carry, on every shape
+// measured on MI355X (256 CUs): as many channels as the workspace layout and
+// the entry count allow. (The reference derives its count from what fits its
+// shared memory, csrc/helix_alltoall.cu:502-535; nothing is staged here.)
 int auto_channels(int cpSize, int entryCount, int cuCount) {
-  int maxCh = max_channel_count(cpSize, cuCount);
-  long slots = static_cast<long>(cuCount) * 32;
-  long c = slots / (static_cast<long>(cpSize) * cpSize);
-  if (c > maxCh) c = maxCh;
+  int c = max_channel_count(cpSize, cuCount);
   if (c > entryCount) c = entryCount;
   if (c < 1) c = 1;
-  return static_cast<int>(c);
+  return c;
 }
 
 int env_channel_count() {

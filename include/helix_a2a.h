@@ -121,9 +121,10 @@ int64_t helix_a2a_workspace_size_per_rank(int cp_size, int cu_count);
 
 /*
  * Channel count an automatic launch would run with for this problem on a
- * device with cu_count compute units (0 = current device). Re-derivation of
- * computeChannelAndGroupCount (csrc/helix_alltoall.cu:486-535) for one
- * wavefront per (sender, receiver, channel) on 256 CUs. Returns -1 on error.
+ * device with cu_count compute units (0 = current device): the counterpart of
+ * computeChannelAndGroupCount (csrc/helix_alltoall.cu:486-535), re-derived for
+ * one wavefront per (sender, receiver, channel) on 256 CUs -- as many channels
+ * as the layout provides and the entries can fill. Returns -1 on error.
  */
 int helix_a2a_auto_channel_count(int cp_size, int entry_count, int cu_count);
 

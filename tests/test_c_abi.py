@@ -62,10 +62,11 @@ def test_known_workspace_sizes_on_256_cus(ops):
 
 
 def test_auto_channel_count(ops):
-    # one wavefront per (sender, receiver, channel): 256 CUs * 32 slots / cp^2, capped by the layout and by the entries
+    # as many channels as the workspace layout provides, never more than there are entries
     assert ops.auto_channel_count(8, 256, 256) == 128
     assert ops.auto_channel_count(8, 5, 256) == 5
-    assert ops.auto_channel_count(16, 1024, 256) == 32
+    assert ops.auto_channel_count(16, 1024, 256) == 64
+    assert ops.auto_channel_count(2, 1000, 256) == 128
     assert ops.auto_channel_count(4, 64, 256) == 64
     assert ops.auto_channel_count(2, 8, 256) == 8
     assert ops.auto_channel_count(8, 0, 256) == 1
