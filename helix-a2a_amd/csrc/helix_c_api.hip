@@ -373,7 +373,8 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, cons
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "no rank descriptors or outputs given");
   if (per_rank[0].cp_size != cp_size || per_rank[0].cp_rank != 0)
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "loopback needs descriptors of ranks 0..cp_size-1 in order");
-  if (stats_mode != HELIX_A2A_STATS_LSE && stats_mode != HELIX_A2A_STATS_MAX_SUM)
+  if (stats_mode != HELIX_A2A_STATS_LSE && stats_mode != HELIX_A2A_STATS_MAX_SUM &&
+      stats_mode != HELIX_A2A_STATS_LSE_PACKED)
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "unknown stats_mode %d", stats_mode);
   if (dtype != HELIX_A2A_DTYPE_BF16 && dtype != HELIX_A2A_DTYPE_FP16)
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "unknown dtype %d", dtype);
@@ -382,7 +383,8 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, cons
   if (rc) return rc;
   KernelArgs& a = plan.args;
   const int x = per_rank[0].send_fields[0].element_count;
-  const int heads = per_rank[0].send_fields[1].element_count / 2;
+  const int statsWidth = per_rank[0].send_fields[1].element_count;
+  const int heads = stats_mode == HELIX_A2A_STATS_LSE_PACKED ? statsWidth : statsWidth / 2;
   if (heads < 1 || x % heads != 0 || (x / heads) % 4 != 0)
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT,
                 "combine needs partial_o rows of heads * head_dim elements with head_dim a multiple of 4 "

@@ -476,9 +476,12 @@ struct OnlineSum {
   __device__ __forceinline__ float inv_total() const { return 1.0f / fmaxf(total, 1e-10f); }
 };
 
-// log-sum-exp of one {stats[2h], stats[2h+1]} pair; NaN and +-inf count as "no contribution"
-__device__ __forceinline__ float lse_of_stats(uint32_t s0, uint32_t s1, int statsMode) {
-  float x = __uint_as_float(s0);
+// log-sum-exp of head h from the 8-byte statistics piece {s0, s1} that holds it;
+// NaN and +-inf count as "no contribution".
+//   mode 0: piece h = {lse, unused}     mode 1: piece h = {running max, running sum}
+//   mode 2: piece h/2 = {lse of head 2*(h/2), lse of head 2*(h/2)+1}
+__device__ __forceinline__ float lse_of_stats(uint32_t s0, uint32_t s1, int statsMode, uint32_t h) {
+  float x = __uint_as_float((statsMode == 2 && (h & 1u)) ? s1 : s0);
   if (statsMode == 1) x = x + fast_log(__uint_as_float(s1));  // running max + ln(running sum)
   return (isnan(x) || isinf(x)) ? -INFINITY : x;
 }
@@ -561,7 +564,7 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
       const uint32_t hB = dataB ? head_of_piece(d.piece0 + 1, a.headMagic) : hA;
       const uint32_t entry = static_cast<uint32_t>(a.entryBegin + ch) + (firstMsg + d.msg) * a.runChannels;
       // where the statistics of heads hA / hB sit: run line and word inside it
-      const uint32_t psA = st.np0 + hA, psB = st.np0 + hB;
+      const uint32_t psA = st.np0 + (a.statsMode == 2 ? hA >> 1 : hA), psB = st.np0 + (a.statsMode == 2 ? hB >> 1 : hB);
       const uint32_t lineA = d.msg * st.lines + psA / kPiecesPerLine, wordA = psA % kPiecesPerLine;
       const uint32_t lineB = d.msg * st.lines + psB / kPiecesPerLine, wordB = psB % kPiecesPerLine;
       // piece B shares the weights of piece A unless it starts the next head
@@ -612,13 +615,13 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
                 const int srcA = static_cast<int>(wordA >> 1);
                 const uint32_t ax = shuffle_from(sv.x, srcA), ay = shuffle_from(sv.y, srcA);
                 const uint32_t az = shuffle_from(sv.z, srcA), aw = shuffle_from(sv.w, srcA);
-                const float la = lse_of_stats((wordA & 1u) ? az : ax, (wordA & 1u) ? aw : ay, a.statsMode);
+                const float la = lse_of_stats((wordA & 1u) ? az : ax, (wordA & 1u) ? aw : ay, a.statsMode, hA);
                 if (takeA) lseA[j] = la;
                 if (anyOwnB) {
                   const int srcB = static_cast<int>(wordB >> 1);
                   const uint32_t bx = shuffle_from(sv.x, srcB), by = shuffle_from(sv.y, srcB);
                   const uint32_t bz = shuffle_from(sv.z, srcB), bw = shuffle_from(sv.w, srcB);
-                  const float lb = lse_of_stats((wordB & 1u) ? bz : bx, (wordB & 1u) ? bw : by, a.statsMode);
+                  const float lb = lse_of_stats((wordB & 1u) ? bz : bx, (wordB & 1u) ? bw : by, a.statsMode, hB);
                   if (takeB) lseB[j] = lb;
                 }
               }

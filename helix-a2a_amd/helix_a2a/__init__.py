@@ -22,7 +22,7 @@ from typing import List, Optional, Sequence, Tuple
 import torch
 
 from helix_a2a import _ops
-from helix_a2a._ops import STATS_LSE, STATS_MAX_SUM  # noqa: F401
+from helix_a2a._ops import STATS_LSE, STATS_LSE_PACKED, STATS_MAX_SUM  # noqa: F401
 from helix_a2a._version import __version__  # noqa: F401
 
 __all__ = [
@@ -34,6 +34,8 @@ __all__ = [
     "alltoall_combine_loopback",
     "STATS_LSE",
     "STATS_MAX_SUM",
+    "STATS_LSE_PACKED",
+    "dcp_a2a_lse_reduce",
 ]
 
 
@@ -123,7 +125,53 @@ def alltoall_combine_loopback(
     Returns ``combined`` (list, rank ``r`` holds ``[E, heads * head_dim]``) or
     ``(combined, lse)`` with ``lse[r]`` of shape ``[E, heads]`` when ``return_lse``.
     ``stats_mode`` says how ``softmax_stats`` pairs encode the weight:
-    ``STATS_LSE`` (slot 0 is the natural-log LSE) or ``STATS_MAX_SUM``
-    (running max, running sum).
+    ``STATS_LSE`` (slot 0 is the natural-log LSE), ``STATS_MAX_SUM`` (running
+    max, running sum) or ``STATS_LSE_PACKED`` (``softmax_stats`` is
+    ``[..., cp_size, heads]`` with one natural-log LSE per head).
     """
     return _ops.alltoall_combine_loopback(partial_o, softmax_stats, workspace, stats_mode, return_lse, channel_count)
+
+
+def dcp_a2a_lse_reduce(
+    cp_attn_out: Sequence[torch.Tensor],
+    cp_attn_lse: Sequence[torch.Tensor],
+    workspace: torch.Tensor,
+    return_lse: bool = False,
+    is_lse_base_on_e: bool = True,
+    channel_count: int = 0,
+):
+    """Combine the partial attention outputs of all logical ranks, as the serving integration does.
+
+    The counterpart of ``dcp_a2a_lse_reduce`` in the reference's vLLM module
+    (patches/dcp_alltoall_helix.py:391-448) for the ``cp_size = len(cp_attn_out)``
+    logical ranks of one device. Rank ``s`` passes ``cp_attn_out[s]`` ``[B, H, D]``
+    (all heads over its KV shard) and ``cp_attn_lse[s]`` ``[B, H]`` fp32; rank ``r``
+    gets back ``[B, H/N, D]``, the exact LSE-weighted combination for its heads
+    ``r*H/N .. (r+1)*H/N - 1``, and with ``return_lse`` the combined LSE ``[B, H/N]``.
+
+    No permute is needed on either side: ``[B, H, D]`` *is* ``[B, N, (H/N)*D]``,
+    which the exchange takes as it is, and the fused combine writes ``[B, H/N, D]``
+    directly (the reference path permutes before and after its kernel,
+    patches/dcp_alltoall_helix.py:545-593).
+    """
+    n = len(cp_attn_out)
+    if n < 1 or len(cp_attn_lse) != n:
+        raise RuntimeError("need one attention output and one LSE tensor per rank")
+    outs, stats = [], []
+    for o, lse in zip(cp_attn_out, cp_attn_lse):
+        if o.dim() != 3 or lse.dim() != 2 or o.shape[:2] != lse.shape or o.size(1) % n != 0:
+            raise RuntimeError("expected cp_attn_out [B, H, D] and cp_attn_lse [B, H] with H divisible by the rank count")
+        b, h, d = o.shape
+        outs.append(o.contiguous().view(b, n, (h // n) * d))
+        lse = lse.contiguous()
+        if not is_lse_base_on_e:
+            lse = lse * 0.6931471805599453  # base-2 LSE -> natural log
+        stats.append(lse.view(b, n, h // n))
+    res = _ops.alltoall_combine_loopback(outs, stats, workspace, STATS_LSE_PACKED, return_lse, channel_count)
+    b, h, d = cp_attn_out[0].shape
+    if return_lse:
+        combined, lses = res
+        if not is_lse_base_on_e:
+            lses = [t * 1.4426950408889634 for t in lses]
+        return [c.view(b, h // n, d) for c in combined], lses
+    return [c.view(b, h // n, d) for c in res]

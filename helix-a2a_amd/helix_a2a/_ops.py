@@ -20,8 +20,9 @@ import torch
 
 MAX_CP_SIZE = 16
 
-STATS_LSE = 0
-STATS_MAX_SUM = 1
+STATS_LSE = 0          # stats pairs: (natural-log LSE, unused)
+STATS_MAX_SUM = 1      # stats pairs: (running max, running sum)
+STATS_LSE_PACKED = 2   # one natural-log LSE per head, no padding
 
 _LIB_NAME = "libhelix_a2a.so"
 
@@ -396,7 +397,8 @@ class CombinePlan:
         cp_size = len(partial_o)
         _require(1 <= cp_size <= MAX_CP_SIZE and len(softmax_stats) == cp_size,
                  "need one partial_o and one softmax_stats tensor per rank")
-        _require(stats_mode in (STATS_LSE, STATS_MAX_SUM), "stats_mode must be STATS_LSE or STATS_MAX_SUM")
+        _require(stats_mode in (STATS_LSE, STATS_MAX_SUM, STATS_LSE_PACKED),
+                 "stats_mode must be STATS_LSE, STATS_MAX_SUM or STATS_LSE_PACKED")
         _check_workspace(workspace, cp_size)
         self.cp_size = cp_size
         self.inputs = (list(partial_o), list(softmax_stats))
@@ -415,7 +417,7 @@ class CombinePlan:
                 shape0 = shape0 or sig
                 _require(sig == shape0, "all ranks must exchange tensors of one shape and dtype")
                 entries, _, x = o3.shape
-                heads = s3.size(-1) // 2
+                heads = s3.size(-1) if stats_mode == STATS_LSE_PACKED else s3.size(-1) // 2
                 _require(x % heads == 0 and (x // heads) % 4 == 0,
                          "partial_o rows must hold heads * head_dim elements, head_dim a multiple of 4")
                 four_d = o.dim() == 4 and o.size(1) == cp_size and o.size(2) == heads

@@ -96,6 +96,8 @@ typedef struct helix_a2a_combine_out {
 /* how softmax_stats encodes the per-(entry, head) weight */
 #define HELIX_A2A_STATS_LSE 0     /* stats[2h] = natural-log LSE, stats[2h+1] ignored (patches/dcp_alltoall_helix.py:560-567) */
 #define HELIX_A2A_STATS_MAX_SUM 1 /* stats[2h] = running max, stats[2h+1] = running sum; LSE = max + ln(sum) */
+#define HELIX_A2A_STATS_LSE_PACKED 2 /* stats[h] = natural-log LSE of head h: the caller's [B, H] LSE tensor as it is
+                                        (patches/dcp_alltoall_helix.py:545-571 pads it to pairs only for the reference kernel) */
 
 /* element type of partial_o for the combine arithmetic */
 #define HELIX_A2A_DTYPE_BF16 0
@@ -175,7 +177,8 @@ int helix_a2a_alltoall_loopback(const helix_a2a_params_t* per_rank, int cp_size,
  * Loopback exchange fused with the LSE-weighted combine: the receive half
  * reduces the cp_size partial outputs of each (entry, head) instead of storing
  * them. recv_fields of per_rank are ignored; out[r] receives rank r's result.
- * heads = send_fields[1].element_count / 2, head_dim = send_fields[0].element_count / heads.
+ * heads = send_fields[1].element_count / 2 (element_count itself for HELIX_A2A_STATS_LSE_PACKED),
+ * head_dim = send_fields[0].element_count / heads.
  */
 int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank,
                                         const helix_a2a_combine_out_t* out, int cp_size,

@@ -257,6 +257,7 @@ def lse_from_stats(stats: np.ndarray, mode: int) -> np.ndarray:
     mode 0: slot 0 is the natural-log LSE, slot 1 unused
             (patches/dcp_alltoall_helix.py:560-567 sends it that way).
     mode 1: (running max, running sum) pairs; LSE = max + ln(sum).
+    (mode 2, one LSE per head without padding, needs no decoding: see combine_after_exchange.)
     """
     stats = np.asarray(stats)
     if mode == 0:
@@ -291,12 +292,16 @@ def combine_after_exchange(recv_o_f32: np.ndarray, recv_stats: np.ndarray, heads
                            dtype=np.float32) -> Tuple[np.ndarray, np.ndarray]:
     """Combine one rank's exchanged tensors.
 
-    recv_o_f32 [E, cp, heads*D] (already widened), recv_stats [E, cp, 2*heads].
-    Returns combined [E, heads*D] and global lse [E, heads].
+    recv_o_f32 [E, cp, heads*D] (already widened), recv_stats [E, cp, 2*heads]
+    (mode 2: [E, cp, heads], the LSE itself). Returns combined [E, heads*D] and global lse [E, heads].
     """
     e, cp, x = recv_o_f32.shape
     d = x // heads
     o = recv_o_f32.reshape(e, cp, heads, d).transpose(1, 0, 2, 3)          # [N, B, H, D]
+    if mode == 2:
+        lse = np.asarray(recv_stats, dtype=dtype).reshape(e, cp, heads).transpose(1, 0, 2)
+        c, g = lse_combine(o, lse, dtype)
+        return c.reshape(e, x), g
     lse = lse_from_stats(np.asarray(recv_stats, dtype=dtype).reshape(e, cp, heads, 2), mode).transpose(1, 0, 2)  # [N, B, H]
     c, g = lse_combine(o, lse, dtype)
     return c.reshape(e, x), g

@@ -212,3 +212,32 @@ def test_combine_while_senders_are_still_writing(hx, ops):
                     assert torch.equal(combined[r], first[r]), f"replay {it} differs on rank {r} with {channels} channels"
     torch.cuda.synchronize()
     assert ops.device_status() == 0
+
+
+@pytest.mark.parametrize("base_e", [True, False])
+def test_dcp_a2a_lse_reduce_matches_the_reference_recipe(hx, ops, base_e):
+    # What the serving integration computes (patches/dcp_alltoall_helix.py:455-504): every rank splits its
+    # [B, H, D] output by head group, the groups are exchanged, and each rank combines its N partials.
+    n, b, h, d = 8, 33, 64, 128
+    ws = workspace(hx, n)
+    g = torch.Generator().manual_seed(21)
+    outs = [torch.randn(b, h, d, generator=g).to(torch.bfloat16).cuda() for _ in range(n)]
+    lses = [(torch.randn(b, h, generator=g) * 4).cuda() for _ in range(n)]
+    lses[3][5, 7] = float("-inf")
+    combined, glse = hx.dcp_a2a_lse_reduce(outs, lses, ws, return_lse=True, is_lse_base_on_e=base_e)
+    torch.cuda.synchronize()
+    assert ops.device_status() == 0
+    hp = h // n
+    assert combined[0].shape == (b, hp, d) and glse[0].shape == (b, hp)
+    o32 = np.stack([ho.bf16_bits_to_f32(torch_bits(t)) for t in outs])          # [N, B, H, D]
+    l32 = np.stack([t.cpu().numpy() for t in lses])                               # [N, B, H]
+    if not base_e:
+        l32 = l32 * np.float32(np.log(2.0))
+    for r in range(n):
+        with np.errstate(all="ignore"):
+            want, want_lse = ho.lse_combine(o32[:, :, r * hp:(r + 1) * hp, :], l32[:, :, r * hp:(r + 1) * hp])
+        if not base_e:
+            want_lse = want_lse / np.float32(np.log(2.0))
+        got = combined[r].float().cpu().numpy()
+        assert (np.abs(got - want) <= ATOL + RTOL * np.abs(want)).all()
+        assert np.allclose(glse[r].cpu().numpy(), want_lse, rtol=1e-4, atol=1e-4)

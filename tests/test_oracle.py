@@ -434,3 +434,14 @@ def test_bf16_widening():
     assert np.array_equal(ho.bf16_bits_to_f32(bits), t.float().numpy())
     h = torch.randn(257).to(torch.float16)
     assert np.array_equal(ho.f16_bits_to_f32(h.view(torch.int16).numpy().view(np.uint16)), h.float().numpy())
+
+
+def test_combine_packed_lse_mode_equals_padded_mode():
+    rng = np.random.default_rng(4)
+    e, cp, heads, d = 3, 4, 6, 8
+    o = rng.standard_normal((e, cp, heads * d)).astype(np.float32)
+    lse = (rng.standard_normal((e, cp, heads)) * 3).astype(np.float32)
+    padded = np.stack((lse, np.zeros_like(lse)), axis=-1).reshape(e, cp, 2 * heads)
+    got2, l2 = ho.combine_after_exchange(o, lse, heads, mode=2)
+    got0, l0 = ho.combine_after_exchange(o, padded, heads, mode=0)
+    assert np.array_equal(got2, got0) and np.array_equal(l2, l0)
