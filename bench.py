@@ -111,6 +111,8 @@ def main() -> int:
     ap.add_argument("--workload", default="c3")
     ap.add_argument("--channels", type=int, default=0, help="0 = automatic")
     ap.add_argument("--combine", action="store_true", help="time the exchange fused with the LSE-weighted combine")
+    ap.add_argument("--graph", type=int, default=0, metavar="G",
+                    help="replay the calls from a captured HIP graph of G calls (steps must be a multiple of G)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
@@ -146,6 +148,17 @@ def main() -> int:
     for _ in range(args.warmup):
         plan.run()
     torch.cuda.synchronize()
+    graph = None
+    if args.graph:
+        if args.steps % args.graph:
+            print("bench.py: --steps must be a multiple of --graph", file=sys.stderr)
+            return 2
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(args.graph):
+                plan.run()
+        graph.replay()
+        torch.cuda.synchronize()
 
     # timed region: exactly K steps between two synchronisations, one HIP event pair around all of
     # them on the launch stream (per-step pairs would put two more commands between every kernel)
@@ -154,8 +167,12 @@ def main() -> int:
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     region_start.record()
-    for _ in range(args.steps):
-        plan.run()
+    if graph is not None:
+        for _ in range(args.steps // args.graph):
+            graph.replay()
+    else:
+        for _ in range(args.steps):
+            plan.run()
     region_end.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
@@ -231,6 +248,7 @@ def main() -> int:
                         + ("exchange fused with the LSE-weighted combine to bf16 [T,H/cp,D]" if args.combine else "exchange only"),
             "cp": w.cp, "T": w.tokens, "H": w.heads, "D": w.head_dim,
             "channels": channels,
+            "launch": f"HIP graph of {args.graph} calls" if args.graph else "eager, one C call per step",
             "algorithmic_bytes_per_call": bytes_per_call,
             "payload_bytes": w.payload_bytes, "wire_bytes": w.wire_bytes,
         },

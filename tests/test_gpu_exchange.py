@@ -528,3 +528,48 @@ def test_receivers_overlapping_their_senders(hx, ops, channels):
     torch.cuda.synchronize()
     assert_clean(ops)
     assert int(bad.item()) == 0
+
+
+# ---------------------------------------------------------------------------
+# graph capture
+# ---------------------------------------------------------------------------
+
+def test_exchange_and_combine_replay_from_a_captured_graph(hx, ops):
+    # The FIFO step counters live in the workspace, not in the kernel arguments, so a captured
+    # launch can be replayed: every replay walks on to the next FIFO entry. Replays are interleaved
+    # with eager work and synchronisations, and every one of them is checked.
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS["c2"]
+    ws = get_workspace(hx, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    plan = ops.LoopbackPlan(ins_o, ins_s, ws)
+    fused = ops.CombinePlan(ins_o, ins_s, ws, ops.STATS_MAX_SUM, return_lse=True)
+    plan.run()
+    fused.run()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        plan.run()
+        fused.run()
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    base_o = [t.clone() for t in ins_o]
+    for replay in range(7):
+        for r in range(w.cp):  # eager work between replays: new payload in the captured buffers
+            ins_o[r].copy_((base_o[r].float() * (1.0 + 0.25 * replay)).to(torch.bfloat16))
+        for t in plan.out_o + plan.out_s + fused.combined:
+            t.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_clean(ops)
+        check_against_oracle(ins_o, ins_s, plan.out_o, plan.out_s, with_numpy=False)
+        # the same graph also ran the fused combine: compare with an eager fused call on the same inputs
+        got = [c.clone() for c in fused.combined]
+        got_lse = [l.clone() for l in fused.lse]
+        eager_c, eager_l = hx.alltoall_combine_loopback(ins_o, ins_s, ws, hx.STATS_MAX_SUM, return_lse=True)
+        torch.cuda.synchronize()
+        for r in range(w.cp):
+            assert torch.equal(got[r], eager_c[r]) and torch.equal(got_lse[r], eager_l[r]), f"replay {replay}, rank {r}"
+    for r in range(w.cp):
+        ins_o[r].copy_(base_o[r])
