@@ -144,7 +144,8 @@ int check_field(const helix_a2a_field_t& f, const char* name, int eltSize, int e
 }
 
 // Validate `count` rank descriptors that share one exchange and build the
-// kernel argument block. `exchangeOutputs` selects whether recv_fields are
+// kernel argument block. Checks that need no device come first, so that a
+// malformed descriptor is reported even where no GPU is present. `exchangeOutputs` selects whether recv_fields are
 // checked (exchange) or ignored (combine).
 int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs, Plan* plan) {
   if (ranks == nullptr || count < 1) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "no rank descriptors given");
@@ -157,18 +158,6 @@ int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs,
   if (p0.workspace == nullptr) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace pointer is null");
   if ((reinterpret_cast<uintptr_t>(p0.workspace) % kUnitBytes) != 0 || (p0.workspace_stride_u64 % 2) != 0)
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace rows must be 16-byte aligned");
-
-  int cuCount = 0;
-  rc = resolve_cu_count(0, &cuCount);
-  if (rc) return rc;
-  const int maxCh = max_channel_count(cp, cuCount);
-  if (p0.max_channel_count != maxCh)
-    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "max_channel_count %d does not match the device's %d (cp_size %d, %d CUs)",
-                p0.max_channel_count, maxCh, cp, cuCount);
-  if (p0.workspace_stride_u64 * 8ull < workspace_bytes(cp, maxCh))
-    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace row of %llu bytes is smaller than the %llu bytes cp_size %d needs",
-                static_cast<unsigned long long>(p0.workspace_stride_u64 * 8ull),
-                static_cast<unsigned long long>(workspace_bytes(cp, maxCh)), cp);
 
   KernelArgs a;
   std::memset(&a, 0, sizeof(a));
@@ -220,6 +209,19 @@ int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs,
   if (sh.lines > kFifoEntryLines)
     return fail(HELIX_A2A_ERR_CAPACITY, "a message of %d bytes needs %d lines, more than one FIFO entry (%d lines)",
                 f0 + f1, sh.lines, kFifoEntryLines);
+
+  // everything above is pure argument checking; from here on the device is consulted
+  int cuCount = 0;
+  rc = resolve_cu_count(0, &cuCount);
+  if (rc) return rc;
+  const int maxCh = max_channel_count(cp, cuCount);
+  if (p0.max_channel_count != maxCh)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "max_channel_count %d does not match the device's %d (cp_size %d, %d CUs)",
+                p0.max_channel_count, maxCh, cp, cuCount);
+  if (p0.workspace_stride_u64 * 8ull < workspace_bytes(cp, maxCh))
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace row of %llu bytes is smaller than the %llu bytes cp_size %d needs",
+                static_cast<unsigned long long>(p0.workspace_stride_u64 * 8ull),
+                static_cast<unsigned long long>(workspace_bytes(cp, maxCh)), cp);
 
   int channels = p0.channel_count > 0 ? p0.channel_count : env_channel_count();
   if (channels > maxCh)

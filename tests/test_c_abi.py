@@ -105,3 +105,88 @@ def test_product_does_not_import_the_oracle():
         text = path.read_text()
         assert "oracle" not in text.lower(), f"{path} mentions the oracle"
         assert "host_model" not in text, f"{path} mentions the test host model"
+
+
+# ---------------------------------------------------------------------------
+# descriptor validation (no device needed: it happens before anything touches the GPU)
+# ---------------------------------------------------------------------------
+
+def _descriptor(ops, cp=4, entries=3, x=128, s=2, rank=0, ptr=0x10000):
+    p = ops._Params()
+    for f, (count, size) in enumerate(((x, 2), (s, 4))):
+        for field in (p.send_fields[f], p.recv_fields[f]):
+            field.data = ptr
+            field.element_count = count
+            field.element_size = size
+            field.stride_bytes = count * size
+    p.entry_count = entries
+    p.workspace = ptr
+    p.workspace_stride_u64 = 1 << 30
+    p.cp_rank, p.cp_size = rank, cp
+    p.channel_count = 0
+    p.max_channel_count = ops.max_channel_count(cp, 256) if 1 <= cp <= 16 else 1
+    return p
+
+
+def _expect_invalid(ops, call, params, count, pattern):
+    import ctypes
+
+    arr = (ops._Params * len(params))(*params)
+    rc = call(arr, count, None) if count is not None else call(ctypes.byref(arr[0]), None)
+    assert rc == 1, f"expected HELIX_A2A_ERR_INVALID_ARGUMENT, got {rc}"
+    msg = ops._lib.helix_a2a_last_error().decode()
+    assert re.search(pattern, msg), msg
+
+
+def test_descriptor_validation_without_a_device(ops):
+    lib = ops._lib
+    send = lib.helix_a2a_alltoall_send
+    cases = [
+        (dict(cp=0), "cp_size"),
+        (dict(cp=17), "cp_size"),
+        (dict(entries=-1), "entry_count"),
+        (dict(rank=4), "cp_rank"),
+        (dict(x=100), "multiple of 16 bytes"),          # 200-byte partial_o rows
+        (dict(s=3), "even|multiple of 8"),              # odd stats width: 12-byte rows
+        (dict(s=0), "positive"),
+        (dict(ptr=0x10004), "aligned"),
+    ]
+    for kwargs, pattern in cases:
+        _expect_invalid(ops, send, [_descriptor(ops, **kwargs)], 1, pattern)
+    p = _descriptor(ops)
+    p.workspace = None
+    _expect_invalid(ops, send, [p], 1, "workspace pointer is null")
+    p = _descriptor(ops)
+    p.send_fields[0].element_size = 4                   # fp32 partial_o
+    _expect_invalid(ops, send, [p], 1, "element size must be 2")
+    p = _descriptor(ops)
+    p.send_fields[1].element_size = 2                   # fp16 stats
+    _expect_invalid(ops, send, [p], 1, "element size must be 4")
+    p = _descriptor(ops)
+    p.send_fields[0].stride_bytes = 100                 # rows overlap
+    _expect_invalid(ops, send, [p], 1, "row stride")
+    p = _descriptor(ops, entries=1 << 20, x=1 << 13)    # 4 * 2^20 rows of 16 KiB
+    _expect_invalid(ops, send, [p], 1, "exceeds 2 GiB")
+    # descriptors of one call must agree and be consecutive ranks
+    a, b = _descriptor(ops, rank=0), _descriptor(ops, rank=1, entries=4)
+    _expect_invalid(ops, send, [a, b], 2, "disagrees")
+    a, b = _descriptor(ops, rank=0), _descriptor(ops, rank=2)
+    _expect_invalid(ops, send, [a, b], 2, "consecutive")
+    a, b = _descriptor(ops, rank=1), _descriptor(ops, rank=1)
+    _expect_invalid(ops, send, [a, b], 2, "twice")
+    _expect_invalid(ops, lib.helix_a2a_alltoall_loopback, [_descriptor(ops, rank=1)], 4, "ranks 0..cp_size-1")
+    _expect_invalid(ops, lib.helix_a2a_alltoall, [_descriptor(ops, x=100)], None, "multiple of 16 bytes")
+    # a message that cannot fit one FIFO entry is a capacity error
+    arr = (ops._Params * 1)(_descriptor(ops, x=61440, s=2))
+    assert send(arr, 1, None) == 3 and "FIFO entry" in lib.helix_a2a_last_error().decode()
+
+
+def test_combine_argument_validation_without_a_device(ops):
+    lib = ops._lib
+    out = (ops._CombineOut * 4)()
+    arr = (ops._Params * 4)(*[_descriptor(ops, rank=r) for r in range(4)])
+    assert lib.helix_a2a_alltoall_combine_loopback(arr, out, 4, 9, 0, None) == 1
+    assert "stats_mode" in lib.helix_a2a_last_error().decode()
+    assert lib.helix_a2a_alltoall_combine_loopback(arr, out, 4, 0, 5, None) == 1
+    assert "dtype" in lib.helix_a2a_last_error().decode()
+    assert lib.helix_a2a_alltoall_combine_loopback(arr, None, 4, 0, 0, None) == 1

@@ -573,3 +573,40 @@ def test_exchange_and_combine_replay_from_a_captured_graph(hx, ops):
             assert torch.equal(got[r], eager_c[r]) and torch.equal(got_lse[r], eager_l[r]), f"replay {replay}, rank {r}"
     for r in range(w.cp):
         ins_o[r].copy_(base_o[r])
+
+
+# ---------------------------------------------------------------------------
+# helix_a2a_alltoall: both halves of one rank in one launch (what one process per GPU would call)
+# ---------------------------------------------------------------------------
+
+def test_single_rank_call_both_halves(hx, ops):
+    import ctypes
+
+    # cp_size 1: the rank is its own peer, the launch sends and receives its own traffic
+    ws = get_workspace(hx, 1)
+    g = torch.Generator().manual_seed(17)
+    o = torch.randn(50, 1, 256, generator=g).to(torch.bfloat16).cuda()
+    s = torch.randn(50, 1, 4, generator=g).cuda()
+    out_o, out_s = torch.empty_like(o), torch.empty_like(s)
+    p = ops._make_params(o, s, out_o, out_s, ws, 0, 1, 0)
+    ops._check(ops._lib.helix_a2a_alltoall(ctypes.byref(p), ops._stream_handle()), "alltoall")
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    assert bits_equal(out_o, o) and bits_equal(out_s, s)
+
+    # cp_size 2 with only rank 0 calling: its receive half waits for rank 1, which never sends;
+    # the bounded wait gives up, the kernel ends normally and the status word says so
+    ws2 = get_workspace(hx, 2, fresh=True)
+    o2 = torch.zeros(3, 2, 64, dtype=torch.bfloat16, device="cuda")
+    s2 = torch.zeros(3, 2, 2, device="cuda")
+    p2 = ops._make_params(o2, s2, torch.empty_like(o2), torch.empty_like(s2), ws2, 0, 2, 1)
+    ops.set_spin_limit_us(0)
+    try:
+        ops._check(ops._lib.helix_a2a_alltoall(ctypes.byref(p2), ops._stream_handle()), "alltoall")
+        torch.cuda.synchronize()
+        status = ops.device_status()
+    finally:
+        ops.set_spin_limit_us(2_000_000)
+    assert status & 1
+    for r in range(2):
+        hx.init_workspace(ws2, r, 2)
