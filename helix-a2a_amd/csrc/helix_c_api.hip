@@ -387,9 +387,9 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, cons
   const int x = per_rank[0].send_fields[0].element_count;
   const int statsWidth = per_rank[0].send_fields[1].element_count;
   const int heads = stats_mode == HELIX_A2A_STATS_LSE_PACKED ? statsWidth : statsWidth / 2;
-  if (heads < 1 || x % heads != 0 || (x / heads) % 4 != 0)
+  if (heads < 1 || x % heads != 0 || (x / heads) % 4 != 0 || x / heads < 32)
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT,
-                "combine needs partial_o rows of heads * head_dim elements with head_dim a multiple of 4 "
+                "combine needs partial_o rows of heads * head_dim elements with head_dim a multiple of 4 and >= 32 "
                 "(row of %d elements, %d heads)", x, heads);
   a.heads = heads;
   a.headDim = x / heads;

@@ -44,6 +44,7 @@ constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any descriptor (extents
 
 constexpr uint32_t kStatusRecvTimeout = 1u;
 constexpr uint32_t kStatusSendTimeout = 2u;
+constexpr uint32_t kStatusInternal = 4u;
 
 // units a lane keeps in flight per chunk of a run
 // (6 x 16 B x 64 lanes = 6 KiB per wavefront; measured best of 3..10 on MI355X)
@@ -413,21 +414,30 @@ __device__ __forceinline__ uint32_t narrow1<1>(float v) {
 // share one layout), loads that unit from each sender's FIFO, and reduces
 // over the senders in registers:
 //   out[e, h, :] = sum_s w[s, h] * partial_o_s[e, h, :],  w = softmax_s(lse[s, h])
-// (patches/dcp_alltoall_helix.py:142-207). The statistics of head h live in
-// piece np0 + h of each message. Every distinct statistics line the lanes of
-// a wavefront need is fetched once per wavefront, by lanes 0..7 in the
-// pattern of a payload line (lane u takes unit u, so the line is validated by
-// its own flag unit in the same load), and handed to the lanes that need it
-// with lane shuffles. The softmax runs online over groups of eight senders,
-// so nothing but two accumulators survives a group. The `parts` wavefronts of
-// a workgroup split the units of a run between them. No LDS, one barrier.
-// The kernel is bounded by instruction issue rather than by memory: exp and
-// ln use the hardware's base-2 units.
+// (patches/dcp_alltoall_helix.py:142-207). The wavefront first acquires the
+// run from every sender through the head token, so every line it touches
+// afterwards is complete.
+//
+// Weights are computed once per wavefront and (message, head), not once per
+// lane: the 64 units of a wave access cover a handful of heads. The lanes that
+// start a head enter it in a slot table (LDS), then the wavefront turns
+// sideways -- lane j serves slot j / G and sender j % G, loads that sender's
+// statistics of that head, and a softmax over the G lanes of a slot gives
+// the weight -- and the weights go back through LDS to the lanes that own
+// units of the head. (G = 4, 8 or 16 lanes per slot for cpSize <= 4, 8, 16.)
+// The `parts` wavefronts of a workgroup split the units of a run.
+constexpr int kCombineSlots = 32;  // distinct (message, head) pairs one wave access may touch
+
 struct CombineCtx {
   __amdgpu_buffer_rsrc_t fifos;  // the whole FIFO region of the receiver's row
   uint32_t channelBase;          // byte offset of sender 0's FIFO of this channel
   uint32_t senderStride;         // bytes between the FIFOs of consecutive senders
   uint32_t stepLo, stepHi;       // lane q: step counter of sender q's stream
+};
+
+struct CombineLds {
+  uint32_t slot[kMaxCombineParts][kCombineSlots][4];          // {first line of the message in the run, head, entry, -}
+  float weight[kMaxCombineParts][kCombineSlots][kMaxCpSize];  // normalised softmax weight per sender
 };
 
 __device__ __forceinline__ uint32_t lane_value(uint32_t v, int q) {
@@ -436,6 +446,7 @@ __device__ __forceinline__ uint32_t lane_value(uint32_t v, int q) {
 __device__ __forceinline__ uint32_t shuffle_from(uint32_t v, int srcLane) {
   return static_cast<uint32_t>(__shfl(static_cast<int>(v), srcLane, kWaveLanes));
 }
+__device__ __forceinline__ float shuffle_xor(float v, int mask) { return __shfl_xor(v, mask, kWaveLanes); }
 
 // byte offset of sender q's open FIFO entry inside the receiver's FIFO region
 __device__ __forceinline__ uint32_t entry_base(const CombineCtx& cx, int q, uint32_t stepLo) {
@@ -443,38 +454,10 @@ __device__ __forceinline__ uint32_t entry_base(const CombineCtx& cx, int q, uint
 }
 
 // exp and ln on the hardware's base-2 units (v_exp_f32 / v_log_f32, about 1 ulp):
-// the combine is bounded by instruction issue, and its result is rounded to
-// 8 mantissa bits anyway. exp(-inf) = 0, ln(0) = -inf, ln(x < 0) = NaN hold.
+// the result is rounded to 8 or 11 mantissa bits anyway. exp(-inf) = 0,
+// ln(0) = -inf, ln(x < 0) = NaN hold.
 __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
 __device__ __forceinline__ float fast_log(float x) { return __builtin_amdgcn_logf(x) * 0.6931471805599453f; }
-
-// Running softmax-weighted sum of one 8-byte piece (4 elements) over the senders.
-struct OnlineSum {
-  float m, total;
-  float acc[4];
-  __device__ __forceinline__ void init() {
-    m = -INFINITY;
-    total = 0.0f;
-    acc[0] = acc[1] = acc[2] = acc[3] = 0.0f;
-  }
-  // raise the running maximum to cover `candidate`
-  __device__ __forceinline__ void rescale(float candidate) {
-    float mNew = fmaxf(m, candidate);
-    float scale = (mNew == -INFINITY) ? 1.0f : fast_exp(m - mNew);  // m == -inf: nothing accumulated yet, scale is 0
-    m = mNew;
-    total *= scale;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) acc[c] *= scale;
-  }
-  __device__ __forceinline__ float weight(float lse) const { return (m == -INFINITY) ? 0.0f : fast_exp(lse - m); }
-  __device__ __forceinline__ void add(float e, const float (&f)[4]) {
-    total += e;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) acc[c] += e * f[c];
-  }
-  __device__ __forceinline__ float lse_value() const { return fast_log(total) + (m == -INFINITY ? 0.0f : m); }
-  __device__ __forceinline__ float inv_total() const { return 1.0f / fmaxf(total, 1e-10f); }
-};
 
 // log-sum-exp of head h from the 8-byte statistics piece {s0, s1} that holds it;
 // NaN and +-inf count as "no contribution".
@@ -487,17 +470,16 @@ __device__ __forceinline__ float lse_of_stats(uint32_t s0, uint32_t s1, int stat
 }
 
 template <int kDtype>
-__device__ __forceinline__ u32x2 narrow_piece(const OnlineSum& o) {
-  const float inv = o.inv_total();
-  u32x2 r = {narrow1<kDtype>(o.acc[0] * inv) | (narrow1<kDtype>(o.acc[1] * inv) << 16),
-             narrow1<kDtype>(o.acc[2] * inv) | (narrow1<kDtype>(o.acc[3] * inv) << 16)};
+__device__ __forceinline__ u32x2 narrow_piece(const float (&acc)[4]) {
+  u32x2 r = {narrow1<kDtype>(acc[0]) | (narrow1<kDtype>(acc[1]) << 16),
+             narrow1<kDtype>(acc[2]) | (narrow1<kDtype>(acc[3]) << 16)};
   return r;
 }
 
-template <int kDtype>
+template <int kDtype, int kLanesPerSlot>
 __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r, int ch, int part, int parts,
-                                                     int lane) {
-  constexpr int kGroup = 8;  // senders whose loads are in flight together
+                                                     int lane, CombineLds& lds) {
+  constexpr int kSlotsPerPass = kWaveLanes / kLanesPerSlot;
   Stream st;
   setup_stream(st, a, 0, ch);
   if (st.msgs == 0) return;  // uniform over the workgroup: same channel
@@ -508,8 +490,7 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
   cx.senderStride = static_cast<uint32_t>(fifo_offset(1, 0, a.maxChannels));
   __amdgpu_buffer_rsrc_t outRsrc = make_rsrc(a.rank[r].recv0, a.recvBytes0);
   __amdgpu_buffer_rsrc_t lseRsrc = make_rsrc(a.rank[r].recv1, a.rank[r].recv1 ? a.recvBytes1 : 0u);
-  const uint32_t piecesPerHead = static_cast<uint32_t>(a.headDim) * 2u / kPieceBytes;
-  const int flagLane = lane | 7;
+  const unsigned long long lanesBelow = (1ull << lane) - 1ull;
 
   // lane q owns the counters of sender q's stream
   int64_t myStep = 0;
@@ -562,130 +543,116 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
       if (__ballot(dataA) == 0ull) continue;  // statistics, padding: nothing to reduce here
       const uint32_t hA = head_of_piece(d.piece0, a.headMagic);
       const uint32_t hB = dataB ? head_of_piece(d.piece0 + 1, a.headMagic) : hA;
+      const bool ownB = dataB && hB != hA;  // the second piece starts the next head
       const uint32_t entry = static_cast<uint32_t>(a.entryBegin + ch) + (firstMsg + d.msg) * a.runChannels;
-      // where the statistics of heads hA / hB sit: run line and word inside it
-      const uint32_t psA = st.np0 + (a.statsMode == 2 ? hA >> 1 : hA), psB = st.np0 + (a.statsMode == 2 ? hB >> 1 : hB);
-      const uint32_t lineA = d.msg * st.lines + psA / kPiecesPerLine, wordA = psA % kPiecesPerLine;
-      const uint32_t lineB = d.msg * st.lines + psB / kPiecesPerLine, wordB = psB % kPiecesPerLine;
-      // piece B shares the weights of piece A unless it starts the next head
-      const bool ownB = dataB && hB != hA;
-      const bool anyOwnB = __ballot(ownB) != 0ull;
 
-      OnlineSum sumA, sumB;
-      sumA.init();
-      sumB.init();
+      // ---- slots: one per distinct (message, head) the lanes of this access touch, in lane order
+      const uint32_t pairA = d.msg * static_cast<uint32_t>(a.heads) + hA;
+      const uint32_t lastPair = dataA ? (ownB ? pairA + 1u : pairA) : 0xFFFFFFFFu;
+      const uint32_t prevPair = shuffle_from(lastPair, lane == 0 ? 0 : lane - 1);
+      const bool newA = dataA && (lane == 0 || prevPair != pairA);
+      const unsigned long long startsA = __ballot(newA), startsB = __ballot(ownB);
+      const int slotA = __popcll(startsA & (lanesBelow | (1ull << lane))) + __popcll(startsB & lanesBelow) - 1;
+      const int slotB = ownB ? slotA + 1 : slotA;
+      const int slotCount = __popcll(startsA) + __popcll(startsB);
+      if (slotCount > kCombineSlots) {  // excluded by the host's shape check (head_dim >= 32)
+        raise_status(a.status, kStatusInternal, lane);
+        return;
+      }
+      if (newA) {
+        lds.slot[part][slotA][0] = d.msg * st.lines;
+        lds.slot[part][slotA][1] = hA;
+        lds.slot[part][slotA][2] = entry;
+      }
+      if (ownB) {
+        lds.slot[part][slotB][0] = d.msg * st.lines;
+        lds.slot[part][slotB][1] = hB;
+        lds.slot[part][slotB][2] = entry;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-      for (int g = 0; g < a.cpSize; g += kGroup) {
-        u32x4 v[kGroup];
-        float lseA[kGroup], lseB[kGroup];
-        SpinGuard guard(a.spinLimitTicks);
-        for (;;) {
-          // payload unit of every sender of the group
+      // ---- weights: lane j serves slot base + j / G and sender j % G
+      for (int base = 0; base < slotCount; base += kSlotsPerPass) {
+        const int slot = base + lane / kLanesPerSlot;
+        const int q = lane % kLanesPerSlot;
+        const bool serving = slot < slotCount && q < a.cpSize;
+        const int slotSafe = slot < kCombineSlots ? slot : 0;
+        const uint32_t msgLine0 = lds.slot[part][slotSafe][0];
+        const uint32_t h = lds.slot[part][slotSafe][1];
+        const uint32_t slotEntry = lds.slot[part][slotSafe][2];
+        const uint32_t ps = st.np0 + (a.statsMode == 2 ? h >> 1 : h);  // statistics piece of head h
+        const uint32_t ls = ps / kPiecesPerLine;
+        const uint32_t word = ps - ls * kPiecesPerLine;
+        const uint32_t qStepLo = shuffle_from(cx.stepLo, q < a.cpSize ? q : 0);
+        const uint32_t off = entry_base(cx, q, qStepLo) + (msgLine0 + ls) * kLineBytes + word * kPieceBytes;
+        const u32x2 sv = __builtin_amdgcn_raw_buffer_load_b64(cx.fifos, serving ? off : kOutOfRange, 0, kAuxSc1);
+        const float lse = serving ? lse_of_stats(sv.x, sv.y, a.statsMode, h) : -INFINITY;
+        float m = lse;
 #pragma unroll
-          for (int j = 0; j < kGroup; ++j) {
-            const int q = g + j;
-            if (q < a.cpSize) {
-              const uint32_t base = entry_base(cx, q, lane_value(cx.stepLo, q));
-              v[j] = __builtin_amdgcn_raw_buffer_load_b128(cx.fifos, live ? base + U * kUnitBytes : kOutOfRange, 0, kAuxSc1);
-            }
-          }
-          // Statistics: every distinct line some lane needs is fetched once per
-          // wavefront, by lanes 0..7 in the pattern of a payload line (lane u takes
-          // unit u, so the line is validated by its own flag unit in the same
-          // load), and handed to the lanes that need it with lane shuffles.
-          bool ok = true;
-          bool pendA = dataA, pendB = ownB;
-          for (;;) {
-            const unsigned long long need = __ballot(pendA || pendB);
-            if (need == 0ull) break;
-            const int leader = __ffsll(static_cast<long long>(need)) - 1;
-            const uint32_t line = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(pendA ? lineA : lineB), leader));
-            const bool takeA = pendA && lineA == line, takeB = pendB && lineB == line;
-            const uint32_t unitOff = line * kLineBytes + static_cast<uint32_t>(lane) * kUnitBytes;
+        for (int x = 1; x < kLanesPerSlot; x <<= 1) m = fmaxf(m, shuffle_xor(m, x));
+        if (m == -INFINITY) m = 0.0f;  // every sender masked: weights 0, lse -inf
+        float e = fast_exp(lse - m);
+        if (isnan(e)) e = 0.0f;
+        float total = e;
 #pragma unroll
-            for (int j = 0; j < kGroup; ++j) {
-              const int q = g + j;
-              if (q < a.cpSize) {
-                const uint32_t sLo = lane_value(cx.stepLo, q), sHi = lane_value(cx.stepHi, q);
-                const uint32_t base = entry_base(cx, q, sLo);
-                const u32x4 sv = __builtin_amdgcn_raw_buffer_load_b128(cx.fifos, lane < 8 ? base + unitOff : kOutOfRange, 0, kAuxSc1);
-                const unsigned long long landed = __ballot(lane != 7 || (sv.z == sLo && sv.w == sHi));
-                ok &= ((landed >> 7) & 1ull) != 0ull;
-                // every lane takes part in every shuffle (a lane can only be read while it is active)
-                const int srcA = static_cast<int>(wordA >> 1);
-                const uint32_t ax = shuffle_from(sv.x, srcA), ay = shuffle_from(sv.y, srcA);
-                const uint32_t az = shuffle_from(sv.z, srcA), aw = shuffle_from(sv.w, srcA);
-                const float la = lse_of_stats((wordA & 1u) ? az : ax, (wordA & 1u) ? aw : ay, a.statsMode, hA);
-                if (takeA) lseA[j] = la;
-                if (anyOwnB) {
-                  const int srcB = static_cast<int>(wordB >> 1);
-                  const uint32_t bx = shuffle_from(sv.x, srcB), by = shuffle_from(sv.y, srcB);
-                  const uint32_t bz = shuffle_from(sv.z, srcB), bw = shuffle_from(sv.w, srcB);
-                  const float lb = lse_of_stats((wordB & 1u) ? bz : bx, (wordB & 1u) ? bw : by, a.statsMode, hB);
-                  if (takeB) lseB[j] = lb;
-                }
-              }
-            }
-            pendA = pendA && !takeA;
-            pendB = pendB && !takeB;
-          }
-          // payload lines: flag unit of each line, shared through a ballot
+        for (int x = 1; x < kLanesPerSlot; x <<= 1) total += shuffle_xor(total, x);
+        if (serving) lds.weight[part][slotSafe][q] = e / fmaxf(total, 1e-10f);
+        // one lane per slot reports the head's combined log-sum-exp
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(fast_log(total) + m), lseRsrc,
+                                              (serving && q == 0) ? (slotEntry * a.heads + h) * 4u : kOutOfRange, 0,
+                                              kAuxNone);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+      // ---- the unit of every sender, weighted
+      const float* wA = lds.weight[part][dataA ? slotA : 0];
+      const float* wB = lds.weight[part][dataA ? slotB : 0];
+      float accA[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      float accB[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      uint32_t flagMismatch = 0u;
+      for (int g = 0; g < a.cpSize; g += 8) {
+        u32x4 v[8];
 #pragma unroll
-          for (int j = 0; j < kGroup; ++j) {
-            const int q = g + j;
-            if (q < a.cpSize) {
-              const uint32_t sLo = lane_value(cx.stepLo, q), sHi = lane_value(cx.stepHi, q);
-              const unsigned long long landed = __ballot(!(live && d.flag) || (v[j].z == sLo && v[j].w == sHi));
-              ok &= ((landed >> flagLane) & 1ull) != 0ull;
-            }
-          }
-          if (__ballot(!ok) == 0ull) break;
-          if (guard.expired()) {
-            raise_status(a.status, kStatusRecvTimeout, lane);
-            return;
-          }
-          __builtin_amdgcn_s_sleep(16);
-          asm volatile("" ::: "memory");
-        }
-        float gmaxA = -INFINITY, gmaxB = -INFINITY;
-#pragma unroll
-        for (int j = 0; j < kGroup; ++j) {
-          if (g + j < a.cpSize) {
-            if (!dataA) lseA[j] = -INFINITY;
-            if (!ownB) lseB[j] = lseA[j];
-            gmaxA = fmaxf(gmaxA, lseA[j]);
-            gmaxB = fmaxf(gmaxB, lseB[j]);
+        for (int j = 0; j < 8; ++j) {
+          const int q = g + j;
+          if (q < a.cpSize) {
+            const uint32_t off = entry_base(cx, q, lane_value(cx.stepLo, q)) + U * kUnitBytes;
+            v[j] = __builtin_amdgcn_raw_buffer_load_b128(cx.fifos, live ? off : kOutOfRange, 0, kAuxSc1);
           }
         }
-        sumA.rescale(gmaxA);
-        sumB.rescale(gmaxB);  // equals gmaxA for every lane whose second piece shares the head
 #pragma unroll
-        for (int j = 0; j < kGroup; ++j) {
-          if (g + j < a.cpSize) {
+        for (int j = 0; j < 8; ++j) {
+          const int q = g + j;
+          if (q < a.cpSize) {
+            const float wa = wA[q], wb = wB[q];
             float f[4];
             u32x2 pa = {v[j].x, v[j].y};
             u32x2 pb = {v[j].z, v[j].w};
-            const float ea = sumA.weight(lseA[j]);
             widen4<kDtype>(pa, f);
-            sumA.add(ea, f);
-            const float eb = anyOwnB ? sumB.weight(lseB[j]) : ea;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) accA[c] += wa * f[c];
             widen4<kDtype>(pb, f);
-            sumB.add(eb, f);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) accB[c] += wb * f[c];
+            if (live && d.flag) flagMismatch |= (v[j].z ^ lane_value(cx.stepLo, q)) | (v[j].w ^ lane_value(cx.stepHi, q));
           }
         }
       }
-      // the lane that holds the first piece of a head reports that head's log-sum-exp
-      const bool reportA = dataA && d.piece0 == hA * piecesPerHead;
-      const bool reportB = dataB && d.piece0 + 1 == hB * piecesPerHead;
-      __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(sumA.lse_value()), lseRsrc,
-                                            reportA ? (entry * a.heads + hA) * 4u : kOutOfRange, 0, kAuxNone);
-      __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(sumB.lse_value()), lseRsrc,
-                                            reportB ? (entry * a.heads + hB) * 4u : kOutOfRange, 0, kAuxNone);
+      if (__ballot(flagMismatch != 0u) != 0ull) {
+        // the head tokens promised complete lines: a flag that disagrees means the workspace is corrupt
+        raise_status(a.status, kStatusInternal, lane);
+        return;
+      }
       const uint32_t rowByte = entry * (st.np0 * kPieceBytes);
-      __builtin_amdgcn_raw_buffer_store_b64(narrow_piece<kDtype>(sumA), outRsrc,
+      __builtin_amdgcn_raw_buffer_store_b64(narrow_piece<kDtype>(accA), outRsrc,
                                             dataA ? rowByte + d.piece0 * kPieceBytes : kOutOfRange, 0, kAuxNone);
-      __builtin_amdgcn_raw_buffer_store_b64(narrow_piece<kDtype>(sumB), outRsrc,
+      __builtin_amdgcn_raw_buffer_store_b64(narrow_piece<kDtype>(accB), outRsrc,
                                             dataB ? rowByte + (d.piece0 + 1) * kPieceBytes : kOutOfRange, 0, kAuxNone);
+      __builtin_amdgcn_wave_barrier();  // the tables are rewritten by the next access
     }
   }
 }
@@ -695,6 +662,7 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
 // rest receive and combine, one workgroup per (receiver, channel).
 template <int kDtype>
 __global__ __launch_bounds__(kMaxCombineParts * kWaveLanes) void helix_combine_kernel(KernelArgs a) {
+  __shared__ CombineLds lds;
   const int parts = static_cast<int>(blockDim.x) / kWaveLanes;
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWaveLanes);
   const int lane = static_cast<int>(threadIdx.x) % kWaveLanes;
@@ -709,7 +677,15 @@ __global__ __launch_bounds__(kMaxCombineParts * kWaveLanes) void helix_combine_k
     return;
   }
   b -= sendBlocks;
-  run_combine_receiver<kDtype>(a, a.rankBegin + b / a.runChannels, b % a.runChannels, wave, parts, lane);
+  const int r = a.rankBegin + b / a.runChannels;
+  const int ch = b % a.runChannels;
+  if (a.cpSize <= 4) {
+    run_combine_receiver<kDtype, 4>(a, r, ch, wave, parts, lane, lds);
+  } else if (a.cpSize <= 8) {
+    run_combine_receiver<kDtype, 8>(a, r, ch, wave, parts, lane, lds);
+  } else {
+    run_combine_receiver<kDtype, 16>(a, r, ch, wave, parts, lane, lds);
+  }
 }
 
 // FIFO region <- 0xFF bytes, info regions <- 0 (csrc/helix_alltoall.cu:637-643).

@@ -418,8 +418,8 @@ class CombinePlan:
                 _require(sig == shape0, "all ranks must exchange tensors of one shape and dtype")
                 entries, _, x = o3.shape
                 heads = s3.size(-1) if stats_mode == STATS_LSE_PACKED else s3.size(-1) // 2
-                _require(x % heads == 0 and (x // heads) % 4 == 0,
-                         "partial_o rows must hold heads * head_dim elements, head_dim a multiple of 4")
+                _require(x % heads == 0 and (x // heads) % 4 == 0 and x // heads >= 32,
+                         "partial_o rows must hold heads * head_dim elements, head_dim a multiple of 4 and >= 32")
                 four_d = o.dim() == 4 and o.size(1) == cp_size and o.size(2) == heads
                 out_shape = (entries, heads, x // heads) if four_d else (entries, x)
                 comb = torch.empty(out_shape, dtype=o.dtype, device=o.device)

@@ -45,6 +45,7 @@ extern "C" {
 /* bits of the device status word (helix_a2a_device_status) */
 #define HELIX_A2A_STATUS_RECV_TIMEOUT 1u /* a receiver gave up polling for a line */
 #define HELIX_A2A_STATUS_SEND_TIMEOUT 2u /* a sender gave up waiting for FIFO room */
+#define HELIX_A2A_STATUS_INTERNAL 4u     /* a kernel met a state its launch checks exclude (corrupt workspace) */
 
 /*
  * One field of a message. Same members and meaning as the reference's
@@ -178,7 +179,7 @@ int helix_a2a_alltoall_loopback(const helix_a2a_params_t* per_rank, int cp_size,
  * reduces the cp_size partial outputs of each (entry, head) instead of storing
  * them. recv_fields of per_rank are ignored; out[r] receives rank r's result.
  * heads = send_fields[1].element_count / 2 (element_count itself for HELIX_A2A_STATS_LSE_PACKED),
- * head_dim = send_fields[0].element_count / heads.
+ * head_dim = send_fields[0].element_count / heads; head_dim must be a multiple of 4 and at least 32.
  */
 int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank,
                                         const helix_a2a_combine_out_t* out, int cp_size,
