@@ -38,6 +38,7 @@ using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
 // sc1 alone is device scope. (The compiler's "volatile" bit 31 would widen
 // the access to system scope; polling loops use a compiler barrier instead.)
 constexpr int kAuxNone = 0;
+constexpr int kAuxNt = 2;  // streaming: received payload is written once and not read again by this kernel
 constexpr int kAuxSc1 = 16;
 constexpr uint32_t kRsrcWord3 = 0x00020000u;   // raw buffer, 32-bit data format
 constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any descriptor (extents are < 2 GiB)
@@ -318,8 +319,8 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
           UnitOffsets o = unit_offsets(st, firstMsg, U, landed[i]);
           u32x2 wa = {v[i].x, v[i].y};
           u32x2 wb = {v[i].z, v[i].w};
-          __builtin_amdgcn_raw_buffer_store_b64(wa, st.field0, o.a0, 0, kAuxNone);
-          __builtin_amdgcn_raw_buffer_store_b64(wb, st.field0, o.b0, 0, kAuxNone);
+          __builtin_amdgcn_raw_buffer_store_b64(wa, st.field0, o.a0, 0, kAuxNt);
+          __builtin_amdgcn_raw_buffer_store_b64(wb, st.field0, o.b0, 0, kAuxNt);
           needField1 |= (o.a1 != kOutOfRange) | (o.b1 != kOutOfRange);
         }
         if (__ballot(needField1) != 0ull) {
@@ -329,8 +330,8 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
             UnitOffsets o = unit_offsets(st, firstMsg, U, landed[i]);
             u32x2 wa = {v[i].x, v[i].y};
             u32x2 wb = {v[i].z, v[i].w};
-            __builtin_amdgcn_raw_buffer_store_b64(wa, st.field1, o.a1, 0, kAuxNone);
-            __builtin_amdgcn_raw_buffer_store_b64(wb, st.field1, o.b1, 0, kAuxNone);
+            __builtin_amdgcn_raw_buffer_store_b64(wa, st.field1, o.a1, 0, kAuxNt);
+            __builtin_amdgcn_raw_buffer_store_b64(wb, st.field1, o.b1, 0, kAuxNt);
           }
         }
         if (__ballot(anyPending) == 0ull) break;
