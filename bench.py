@@ -22,7 +22,7 @@ import time
 from pathlib import Path
 
 ROOT = Path(__file__).resolve().parent
-for _p in (ROOT / "helix-a2a_amd", ROOT, ROOT / "tests"):
+for _p in (ROOT / "helix-a2a_amd", ROOT):
     if str(_p) not in sys.path:
         sys.path.insert(0, str(_p))
 
@@ -50,7 +50,6 @@ def cpu_baseline(w, budget_s: float = 12.0):
     import torch
 
     from helix_a2a.workloads import make_inputs
-    from helix_testing import torch_bits
     from oracle import helix_oracle as ho
 
     ins_o, ins_s = make_inputs(w, "cpu")
@@ -76,7 +75,7 @@ def cpu_baseline(w, budget_s: float = 12.0):
     ws = model.new_workspace(w.cp, sm)
     for r in range(w.cp):
         model.init_workspace(ws, r, w.cp, sm)
-    np_o, np_s = [torch_bits(t) for t in ins_o], [torch_bits(t) for t in ins_s]
+    np_o, np_s = [ho.torch_bits(t) for t in ins_o], [ho.torch_bits(t) for t in ins_s]
     model_times = []
     t_end = time.perf_counter() + budget_s * 0.4
     while len(model_times) < 3 or (time.perf_counter() < t_end and len(model_times) < 20):
@@ -197,11 +196,10 @@ def main() -> int:
     if not args.no_check and args.combine:
         import numpy as np
 
-        from helix_testing import torch_bits
         combined = plan.run()
         torch.cuda.synchronize()
-        recv_o = ho.exchange_closed_form([torch_bits(t) for t in ins_o])
-        recv_s = ho.exchange_closed_form([torch_bits(t) for t in ins_s])
+        recv_o = ho.exchange_closed_form([ho.torch_bits(t) for t in ins_o])
+        recv_s = ho.exchange_closed_form([ho.torch_bits(t) for t in ins_s])
         for r in range(w.cp):
             with np.errstate(all="ignore"):
                 want, _ = ho.combine_after_exchange(ho.bf16_bits_to_f32(recv_o[r]), recv_s[r].view(np.float32),

@@ -168,6 +168,8 @@ def initialize_workspace(workspace: torch.Tensor, cp_rank: int, cp_size: int) ->
     need = get_workspace_size_per_rank(cp_size)
     _require(workspace.size(1) * 8 >= need, f"workspace rows hold {workspace.size(1) * 8} bytes, {need} needed")
     row_ptr = workspace.data_ptr() + cp_rank * workspace.stride(0) * 8
+    # a reset starts a new epoch: half-finished exchanges of logical ranks on this workspace are void
+    _groups.pop((workspace.device.index or 0, workspace.data_ptr(), cp_size), None)
     with torch.cuda.device(workspace.device):
         _check(_lib.helix_a2a_init_workspace(row_ptr, cp_size, 0, _stream_handle()), "init_workspace")
 

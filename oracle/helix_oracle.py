@@ -243,6 +243,15 @@ def exchange_single_copy(inputs):
 # combine
 # ---------------------------------------------------------------------------
 
+def torch_bits(t) -> np.ndarray:
+    """Raw bit pattern of a torch tensor as an unsigned numpy array (bf16/fp16 -> uint16, fp32 -> uint32)."""
+    import torch
+
+    t = t.detach().cpu().contiguous()
+    view = {2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()]
+    return t.view(view).numpy().view(_uint_of(t.view(view).numpy()))
+
+
 def bf16_bits_to_f32(bits: np.ndarray) -> np.ndarray:
     return (bits.astype(np.uint32) << 16).view(np.float32)
 

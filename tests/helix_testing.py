@@ -107,13 +107,10 @@ class HostModel:
 # ---------------------------------------------------------------------------
 
 def torch_bits(t) -> np.ndarray:
-    """Raw bit pattern of a torch tensor as an unsigned numpy array (bf16/fp16 -> uint16, fp32 -> uint32)."""
-    import torch
+    """Raw bit pattern of a torch tensor as an unsigned numpy array (see oracle.helix_oracle.torch_bits)."""
+    from oracle.helix_oracle import torch_bits as impl
 
-    t = t.detach().cpu().contiguous()
-    view = {2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()]
-    unsigned = {2: np.uint16, 4: np.uint32, 8: np.uint64}[t.element_size()]
-    return t.view(view).numpy().view(unsigned)
+    return impl(t)
 
 
 def coded_inputs(cp: int, entries: int, x: int, s: int) -> Tuple[List[np.ndarray], List[np.ndarray]]:
