@@ -69,6 +69,13 @@ def cpu_baseline(w, budget_s: float = 12.0):
             break
     times.sort()
     p50 = percentile(times, 0.5)
+    single = []
+    for _ in range(10):
+        t0 = time.perf_counter()
+        ho.exchange_single_copy(ins_o)
+        ho.exchange_single_copy(ins_s)
+        single.append(time.perf_counter() - t0)
+    single.sort()
     # 2) the C restatement of the reference kernel (its FIFO + LL128 algorithm), one thread, a few calls
     model = ho.RefModel()
     sm = 16
@@ -94,6 +101,7 @@ def cpu_baseline(w, budget_s: float = 12.0):
         "sample": (f"{len(times)} calls of the torch-CPU transpose/hand-off/transpose exchange of workload {w.name} "
                    f"(all {w.cp} ranks, bf16+fp32), p50; GB/s uses the GPU path's algorithmic bytes so the ratio "
                    f"is a time ratio"),
+        "single_strided_copy_us_per_call": percentile(single, 0.5) * 1e6,
         "reference_kernel_model": {
             "us_per_call": m50 * 1e6,
             "cores": 1,
@@ -110,6 +118,9 @@ def main() -> int:
     ap.add_argument("--workload", default="c3")
     ap.add_argument("--channels", type=int, default=0, help="0 = automatic")
     ap.add_argument("--combine", action="store_true", help="time the exchange fused with the LSE-weighted combine")
+    ap.add_argument("--layout", choices=("token", "head"), default="token",
+                    help="token: one entry per token, messages of H/cp heads (default); head: one entry per "
+                         "(token, head), stats are one float2 -- the layout the reference's serving integration passes")
     ap.add_argument("--graph", type=int, default=0, metavar="G",
                     help="replay the calls from a captured HIP graph of G calls (steps must be a multiple of G)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -126,7 +137,7 @@ def main() -> int:
 
     import helix_a2a
     from helix_a2a import _ops
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_a2a.workloads import WORKLOADS, as_head_layout, make_inputs
     from oracle import helix_oracle as ho
 
     if not torch.cuda.is_available():
@@ -138,11 +149,22 @@ def main() -> int:
     for r in range(w.cp):
         helix_a2a.init_workspace(ws, r, w.cp)
     ins_o, ins_s = make_inputs(w, "cuda")
+    entries = w.tokens
+    bytes_exchange, bytes_combine = w.exchange_bytes, w.combine_bytes
+    if args.layout == "head":
+        if args.combine:
+            print("bench.py: --combine is measured on the token layout", file=sys.stderr)
+            return 2
+        pairs = [as_head_layout(w, o, s) for o, s in zip(ins_o, ins_s)]
+        ins_o, ins_s = [p[0] for p in pairs], [p[1] for p in pairs]
+        entries = w.tokens * w.heads_per_rank
+        msg = 2 * w.head_dim + 8
+        bytes_exchange = w.cp * w.cp * entries * (2 * msg + 2 * 128 * (-(-msg // 120)))
     if args.combine:
         plan = _ops.CombinePlan(ins_o, ins_s, ws, _ops.STATS_MAX_SUM, False, args.channels)
     else:
         plan = _ops.LoopbackPlan(ins_o, ins_s, ws, args.channels)
-    channels = args.channels or _ops.auto_channel_count(w.cp, w.tokens)
+    channels = args.channels or _ops.auto_channel_count(w.cp, entries)
 
     for _ in range(args.warmup):
         plan.run()
@@ -178,7 +200,7 @@ def main() -> int:
     status = _ops.device_status()
     avg_kernel_ms = region_start.elapsed_time(region_end) / args.steps  # launch-to-launch, gaps included
     ms_per_step = wall * 1e3 / args.steps
-    bytes_per_call = w.combine_bytes if args.combine else w.exchange_bytes
+    bytes_per_call = bytes_combine if args.combine else bytes_exchange
 
     # distribution of single calls (event pair per call), outside the timed region
     n_dist = min(args.steps, 500)
@@ -243,7 +265,8 @@ def main() -> int:
         "config": {
             "workload": f"{w.name}: Helix a2a loopback, cp={w.cp} logical ranks, T={w.tokens}, H={w.heads}, D={w.head_dim}, "
                         f"partial_o bf16 [T,cp,H/cp,D] + softmax_stats fp32 [T,cp,H/cp,2], "
-                        + ("exchange fused with the LSE-weighted combine to bf16 [T,H/cp,D]" if args.combine else "exchange only"),
+                        + ("exchange fused with the LSE-weighted combine to bf16 [T,H/cp,D]" if args.combine else "exchange only")
+                        + (", passed per head as [T*H/cp, cp, D] + [T*H/cp, cp, 2]" if args.layout == "head" else ""),
             "cp": w.cp, "T": w.tokens, "H": w.heads, "D": w.head_dim,
             "channels": channels,
             "launch": f"HIP graph of {args.graph} calls" if args.graph else "eager, one C call per step",
@@ -266,10 +289,10 @@ def main() -> int:
             "peak": PEAK_HBM_GBPS,
             "unit": "GB/s",
             "frac": achieved / PEAK_HBM_GBPS,
-            "traffic": None if args.combine else MEASURED_TRAFFIC_BYTES.get((w.name, channels)),
+            "traffic": None if (args.combine or args.layout == "head") else MEASURED_TRAFFIC_BYTES.get((w.name, channels)),
         },
     }
-    if not args.no_cpu_baseline and not args.combine:
+    if not args.no_cpu_baseline and not args.combine and args.layout == "token":
         result["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(result))
     return 0 if ok else 1
