@@ -610,3 +610,29 @@ def test_single_rank_call_both_halves(hx, ops):
     assert status & 1
     for r in range(2):
         hx.init_workspace(ws2, r, 2)
+
+
+# ---------------------------------------------------------------------------
+# nothing to exchange: zero entries is a valid call that launches nothing
+# ---------------------------------------------------------------------------
+
+def test_empty_inputs(hx, ops):
+    cp = 4
+    ws = get_workspace(hx, cp)
+    o = [torch.empty(0, cp, 256, dtype=torch.bfloat16, device="cuda") for _ in range(cp)]
+    s = [torch.empty(0, cp, 2, device="cuda") for _ in range(cp)]
+    out_o, out_s = hx.alltoall_loopback(o, s, ws)
+    assert all(t.shape == (0, cp, 256) for t in out_o) and all(t.shape == (0, cp, 2) for t in out_s)
+    outs = [hx.alltoall(o[r], s[r], ws, cp_rank=r, cp_size=cp) for r in range(cp)]
+    assert all(a.shape == (0, cp, 256) and b.shape == (0, cp, 2) for a, b in outs)
+    combined = hx.alltoall_combine_loopback(o, s, ws, hx.STATS_LSE_PACKED)
+    assert all(t.shape[0] == 0 for t in combined)
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    # the workspace was not touched: a real exchange right after still works
+    g = torch.Generator().manual_seed(3)
+    o1 = [torch.randn(5, cp, 256, generator=g).to(torch.bfloat16).cuda() for _ in range(cp)]
+    s1 = [torch.randn(5, cp, 2, generator=g).cuda() for _ in range(cp)]
+    got_o, got_s = hx.alltoall_loopback(o1, s1, ws)
+    torch.cuda.synchronize()
+    check_against_oracle(o1, s1, got_o, got_s)
