@@ -241,3 +241,47 @@ def test_dcp_a2a_lse_reduce_matches_the_reference_recipe(hx, ops, base_e):
         got = combined[r].float().cpu().numpy()
         assert (np.abs(got - want) <= ATOL + RTOL * np.abs(want)).all()
         assert np.allclose(glse[r].cpu().numpy(), want_lse, rtol=1e-4, atol=1e-4)
+
+
+# ---------------------------------------------------------------------------
+# the pipeline benchmark's three formulations agree, eagerly and from captured graphs
+# ---------------------------------------------------------------------------
+
+def _load_pipeline_benchmark():
+    import importlib.util
+    import os
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "helix-a2a_amd", "benchmark",
+                        "benchmark_helix_pipeline.py")
+    spec = importlib.util.spec_from_file_location("benchmark_helix_pipeline", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def test_pipeline_benchmark_formulations_agree(hx, ops):
+    pb = _load_pipeline_benchmark()
+    n, b, h, d = 4, 16, 32, 128
+    ws = workspace(hx, n)
+    g = torch.Generator().manual_seed(77)
+    outs = [torch.randn(b, h, d, generator=g).to(torch.bfloat16).cuda() for _ in range(n)]
+    lses = [(torch.randn(b, h, generator=g).abs() + 1.0).cuda() for _ in range(n)]
+    lses[1][3, 5] = float("-inf")                      # a masked shard
+    # the benchmark's torch combine against the oracle's fp64 combine
+    want = ho.lse_combine(np.stack([ho.bf16_bits_to_f32(torch_bits(o)) for o in outs]),
+                          np.stack([l.cpu().numpy() for l in lses]), dtype=np.float64)[0]    # [B, H, D]
+    off = pb.Stages(False)
+    for name in ("dcp", "recipe", "fused"):
+        got = pb.PIPELINES[name](outs, lses, ws, off)
+        torch.cuda.synchronize()
+        for r in range(n):
+            ref = want[:, r * (h // n):(r + 1) * (h // n), :]
+            err = np.abs(got[r].float().cpu().numpy() - ref)
+            assert (err <= 2e-2 + 2e-2 * np.abs(ref)).all(), f"{name}: rank {r} off by {err.max()}"
+    # each pipeline replays from a captured graph and the timer returns sane figures
+    for name in ("recipe", "fused"):
+        res = pb.bench_graph(pb.PIPELINES[name], outs, lses, ws, warmup=2, iters=5)
+        assert 0 < res["total"]["p50"] < 1e5
+    res = pb.bench_eager(pb.pipeline_recipe, outs, lses, ws, warmup=1, iters=3)
+    assert set(res) == {"total", "copy", "a2a", "combine"}
+    assert ops.device_status() == 0
