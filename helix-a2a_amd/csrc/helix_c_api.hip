@@ -423,11 +423,9 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, cons
     long parts = cover < fill ? cover : fill;
     if (parts < 1) parts = 1;
     if (parts > kMaxCombineParts) parts = kMaxCombineParts;
-    int p2 = 1;
-    while (p2 * 2 <= parts) p2 *= 2;
     a.doSend = 1;
     a.doRecv = 1;
-    HELIX_HIP_TRY(launch_combine(a, p2, static_cast<hipStream_t>(stream)));
+    HELIX_HIP_TRY(launch_combine(a, static_cast<int>(parts), static_cast<hipStream_t>(stream)));
   }
   return HELIX_A2A_OK;
 }

@@ -43,13 +43,22 @@ constexpr int kAuxSc1 = 16;
 constexpr uint32_t kRsrcWord3 = 0x00020000u;   // raw buffer, 32-bit data format
 constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any descriptor (extents are < 2 GiB)
 
+// Both kernels are held to four wavefronts per SIMD (16 per CU): with more
+// resident wavefronts the same traffic takes 1-5 % longer on MI355X, on every
+// shape measured, whatever the register count would allow.
+#define HELIX_WAVES_PER_SIMD __attribute__((amdgpu_waves_per_eu(4, 4)))
+
 constexpr uint32_t kStatusRecvTimeout = 1u;
 constexpr uint32_t kStatusSendTimeout = 2u;
 constexpr uint32_t kStatusInternal = 4u;
 
-// units a lane keeps in flight per chunk of a run
-// (6 x 16 B x 64 lanes = 6 KiB per wavefront; measured best of 3..10 on MI355X)
-constexpr int kUnitsInFlight = 6;
+// Units a lane keeps in flight per pass over a run: at most kMaxUnitsInFlight
+// (6 x 16 B x 64 lanes = 6 KiB per wavefront), and no more than the runs of a
+// launch need -- the host picks the count (units_in_flight_for_run) so that a
+// run takes the fewest passes and no pass issues accesses that every lane
+// opts out of. The count is a template parameter of the wave programs, so the
+// units stay in registers; the kernels branch once, wave-uniformly, on
+// KernelArgs::unitsInFlight.
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), kRsrcWord3);
@@ -143,7 +152,7 @@ __device__ __forceinline__ UnitOffsets unit_offsets(const Stream& st, uint32_t f
 // ---------------------------------------------------------------------------
 // sender
 // ---------------------------------------------------------------------------
-template <int kAux>
+template <int kAux, int kUnitsInFlight>
 __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, int ch, int lane) {
   Stream st;
   setup_stream(st, a, r, ch);
@@ -222,7 +231,7 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
 // ---------------------------------------------------------------------------
 // receiver
 // ---------------------------------------------------------------------------
-template <int kAux>
+template <int kAux, int kUnitsInFlight>
 __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, int ch, int lane) {
   Stream st;
   setup_stream(st, a, s, ch);
@@ -350,11 +359,24 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
   }
 }
 
+// The one wave-uniform branch on the units-in-flight count of the launch.
+template <int kAux>
+__device__ __forceinline__ void run_sender_any(const KernelArgs& a, int s, int r, int ch, int lane) {
+  switch (a.unitsInFlight) {
+    case 1: run_sender<kAux, 1>(a, s, r, ch, lane); break;
+    case 2: run_sender<kAux, 2>(a, s, r, ch, lane); break;
+    case 3: run_sender<kAux, 3>(a, s, r, ch, lane); break;
+    case 4: run_sender<kAux, 4>(a, s, r, ch, lane); break;
+    case 5: run_sender<kAux, 5>(a, s, r, ch, lane); break;
+    default: run_sender<kAux, kMaxUnitsInFlight>(a, s, r, ch, lane); break;
+  }
+}
 // Wavefront w of a launch: sender wavefronts come first in dispatch order so
 // that no receiver can occupy a slot a not-yet-started sender needs.
 // Within a direction, w = (local rank * runChannels + channel) * cp + peer:
 // neighbouring wavefronts touch neighbouring rows of the same entry.
-__global__ __launch_bounds__(kBlockThreads) void helix_exchange_kernel(KernelArgs a) {
+template <int kUnitsInFlight>
+__global__ __launch_bounds__(kBlockThreads) HELIX_WAVES_PER_SIMD void helix_exchange_kernel(KernelArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWaveLanes);
   const int lane = static_cast<int>(threadIdx.x) % kWaveLanes;
   int w = static_cast<int>(blockIdx.x) * kWavesPerBlock + wave;
@@ -369,9 +391,9 @@ __global__ __launch_bounds__(kBlockThreads) void helix_exchange_kernel(KernelArg
   const int ch = t % a.runChannels;
   const int local = a.rankBegin + t / a.runChannels;
   if (isSender) {
-    run_sender<kAuxSc1>(a, local, peer, ch, lane);
+    run_sender<kAuxSc1, kUnitsInFlight>(a, local, peer, ch, lane);
   } else {
-    run_receiver<kAuxSc1>(a, local, peer, ch, lane);
+    run_receiver<kAuxSc1, kUnitsInFlight>(a, local, peer, ch, lane);
   }
 }
 
@@ -547,6 +569,27 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
       const bool ownB = dataB && hB != hA;  // the second piece starts the next head
       const uint32_t entry = static_cast<uint32_t>(a.entryBegin + ch) + (firstMsg + d.msg) * a.runChannels;
 
+      // Up to eight senders: their unit loads go out before the weights are
+      // worked out -- they do not depend on them, and the two round trips
+      // overlap. (With sixteen, holding the first eight units that long costs a
+      // quarter of the resident wavefronts, which costs more than it saves.)
+      // Senders beyond cpSize are read out of range (zeros, no memory traffic),
+      // which keeps the sequence free of branches.
+      constexpr bool kLoadUnitsEarly = kLanesPerSlot <= 8;
+      u32x4 v[8];
+      auto load_units = [&](int g) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int q = g + j;
+          if (q < kLanesPerSlot) {
+            const int qs = q < a.cpSize ? q : 0;
+            const uint32_t off = entry_base(cx, qs, lane_value(cx.stepLo, qs)) + U * kUnitBytes;
+            v[j] = __builtin_amdgcn_raw_buffer_load_b128(cx.fifos, (live && q < a.cpSize) ? off : kOutOfRange, 0, kAuxSc1);
+          }
+        }
+      };
+      if (kLoadUnitsEarly) load_units(0);
+
       // ---- slots: one per distinct (message, head) the lanes of this access touch, in lane order
       const uint32_t pairA = d.msg * static_cast<uint32_t>(a.heads) + hA;
       const uint32_t lastPair = dataA ? (ownB ? pairA + 1u : pairA) : 0xFFFFFFFFu;
@@ -615,21 +658,16 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
       float accA[4] = {0.0f, 0.0f, 0.0f, 0.0f};
       float accB[4] = {0.0f, 0.0f, 0.0f, 0.0f};
       uint32_t flagMismatch = 0u;
-      for (int g = 0; g < a.cpSize; g += 8) {
-        u32x4 v[8];
+#pragma unroll 1  // sixteen senders: one group of eight units in registers at a time
+      for (int g = 0; g < kLanesPerSlot; g += 8) {
+        if (g > 0 || !kLoadUnitsEarly) load_units(g);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const int q = g + j;
-          if (q < a.cpSize) {
-            const uint32_t off = entry_base(cx, q, lane_value(cx.stepLo, q)) + U * kUnitBytes;
-            v[j] = __builtin_amdgcn_raw_buffer_load_b128(cx.fifos, live ? off : kOutOfRange, 0, kAuxSc1);
-          }
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int q = g + j;
-          if (q < a.cpSize) {
-            const float wa = wA[q], wb = wB[q];
+          if (q < kLanesPerSlot) {
+            const bool have = q < a.cpSize;
+            const int qs = have ? q : 0;
+            const float wa = have ? wA[q] : 0.0f, wb = have ? wB[q] : 0.0f;
             float f[4];
             u32x2 pa = {v[j].x, v[j].y};
             u32x2 pb = {v[j].z, v[j].w};
@@ -639,7 +677,8 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
             widen4<kDtype>(pb, f);
 #pragma unroll
             for (int c = 0; c < 4; ++c) accB[c] += wb * f[c];
-            if (live && d.flag) flagMismatch |= (v[j].z ^ lane_value(cx.stepLo, q)) | (v[j].w ^ lane_value(cx.stepHi, q));
+            if (live && d.flag && have)
+              flagMismatch |= (v[j].z ^ lane_value(cx.stepLo, qs)) | (v[j].w ^ lane_value(cx.stepHi, qs));
           }
         }
       }
@@ -661,8 +700,8 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
 // Workgroups of `parts` wavefronts (blockDim.x / 64). The first
 // ceil(senderStreams / parts) workgroups send, one stream per wavefront; the
 // rest receive and combine, one workgroup per (receiver, channel).
-template <int kDtype>
-__global__ __launch_bounds__(kMaxCombineParts * kWaveLanes) void helix_combine_kernel(KernelArgs a) {
+template <int kDtype, int kLanesPerSlot>
+__global__ __launch_bounds__(kMaxCombineParts * kWaveLanes) HELIX_WAVES_PER_SIMD void helix_combine_kernel(KernelArgs a) {
   __shared__ CombineLds lds;
   const int parts = static_cast<int>(blockDim.x) / kWaveLanes;
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWaveLanes);
@@ -674,19 +713,13 @@ __global__ __launch_bounds__(kMaxCombineParts * kWaveLanes) void helix_combine_k
     const int w = b * parts + wave;
     if (w >= senderStreams) return;
     const int t = w / a.cpSize;
-    run_sender<kAuxSc1>(a, a.rankBegin + t / a.runChannels, w % a.cpSize, t % a.runChannels, lane);
+    run_sender_any<kAuxSc1>(a, a.rankBegin + t / a.runChannels, w % a.cpSize, t % a.runChannels, lane);
     return;
   }
   b -= sendBlocks;
   const int r = a.rankBegin + b / a.runChannels;
   const int ch = b % a.runChannels;
-  if (a.cpSize <= 4) {
-    run_combine_receiver<kDtype, 4>(a, r, ch, wave, parts, lane, lds);
-  } else if (a.cpSize <= 8) {
-    run_combine_receiver<kDtype, 8>(a, r, ch, wave, parts, lane, lds);
-  } else {
-    run_combine_receiver<kDtype, 16>(a, r, ch, wave, parts, lane, lds);
-  }
+  run_combine_receiver<kDtype, kLanesPerSlot>(a, r, ch, wave, parts, lane, lds);
 }
 
 // FIFO region <- 0xFF bytes, info regions <- 0 (csrc/helix_alltoall.cu:637-643).
@@ -701,27 +734,53 @@ __global__ __launch_bounds__(256) void helix_init_row_kernel(u32x4* row, uint64_
 
 }  // namespace
 
-hipError_t launch_exchange(const KernelArgs& a, hipStream_t stream) {
+// The largest run of the launch is the first one of channel 0's streams.
+static KernelArgs with_units_in_flight(KernelArgs a) {
+  const MsgShape sh = make_msg_shape(a.field0Bytes, a.field1Bytes);
+  const int msgs = stream_msg_count(a.entryBegin, a.entryEnd, 0, a.runChannels);
+  const int perEntry = msgs_per_fifo_entry(sh);
+  a.unitsInFlight = units_in_flight_for_run(static_cast<long>(msgs < perEntry ? msgs : perEntry) * sh.units);
+  return a;
+}
+
+hipError_t launch_exchange(const KernelArgs& args, hipStream_t stream) {
+  const KernelArgs a = with_units_in_flight(args);
   int directions = (a.doSend ? 1 : 0) + (a.doRecv ? 1 : 0);
   int waves = directions * waves_per_direction(a);
   if (waves <= 0) return hipSuccess;
   int blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
-  hipLaunchKernelGGL(helix_exchange_kernel, dim3(blocks), dim3(kBlockThreads), 0, stream, a);
+  switch (a.unitsInFlight) {
+    case 1: hipLaunchKernelGGL(helix_exchange_kernel<1>, dim3(blocks), dim3(kBlockThreads), 0, stream, a); break;
+    case 2: hipLaunchKernelGGL(helix_exchange_kernel<2>, dim3(blocks), dim3(kBlockThreads), 0, stream, a); break;
+    case 3: hipLaunchKernelGGL(helix_exchange_kernel<3>, dim3(blocks), dim3(kBlockThreads), 0, stream, a); break;
+    case 4: hipLaunchKernelGGL(helix_exchange_kernel<4>, dim3(blocks), dim3(kBlockThreads), 0, stream, a); break;
+    case 5: hipLaunchKernelGGL(helix_exchange_kernel<5>, dim3(blocks), dim3(kBlockThreads), 0, stream, a); break;
+    default: hipLaunchKernelGGL(helix_exchange_kernel<kMaxUnitsInFlight>, dim3(blocks), dim3(kBlockThreads), 0, stream, a); break;
+  }
   return hipGetLastError();
 }
 
-hipError_t launch_combine(const KernelArgs& a, int parts, hipStream_t stream) {
+hipError_t launch_combine(const KernelArgs& args, int parts, hipStream_t stream) {
+  const KernelArgs a = with_units_in_flight(args);
   const int senderStreams = a.doSend ? a.rankCount * a.runChannels * a.cpSize : 0;
   if (a.rankCount * a.runChannels <= 0) return hipSuccess;
   if (parts < 1) parts = 1;
   if (parts > kMaxCombineParts) parts = kMaxCombineParts;
   const int blocks = (senderStreams + parts - 1) / parts + a.rankCount * a.runChannels;
   dim3 block(static_cast<unsigned>(parts * kWaveLanes));
+  // lanes per slot of the sideways pass: the smallest of 4, 8, 16 that holds every sender
+  const int g = a.cpSize <= 4 ? 4 : a.cpSize <= 8 ? 8 : 16;
+#define HELIX_LAUNCH_COMBINE(DT, G) hipLaunchKernelGGL((helix_combine_kernel<DT, G>), dim3(blocks), block, 0, stream, a)
   if (a.dtype == 1) {
-    hipLaunchKernelGGL(helix_combine_kernel<1>, dim3(blocks), block, 0, stream, a);
+    if (g == 4) HELIX_LAUNCH_COMBINE(1, 4);
+    else if (g == 8) HELIX_LAUNCH_COMBINE(1, 8);
+    else HELIX_LAUNCH_COMBINE(1, 16);
   } else {
-    hipLaunchKernelGGL(helix_combine_kernel<0>, dim3(blocks), block, 0, stream, a);
+    if (g == 4) HELIX_LAUNCH_COMBINE(0, 4);
+    else if (g == 8) HELIX_LAUNCH_COMBINE(0, 8);
+    else HELIX_LAUNCH_COMBINE(0, 16);
   }
+#undef HELIX_LAUNCH_COMBINE
   return hipGetLastError();
 }
 

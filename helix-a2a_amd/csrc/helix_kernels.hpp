@@ -35,6 +35,7 @@ struct KernelArgs {
   uint32_t lineMagic;               // line_div_magic(lines per message)
   int rankBegin, rankCount;
   int doSend, doRecv;
+  int unitsInFlight;        // units_in_flight_for_run(largest run of the launch), 1..kMaxUnitsInFlight
   uint64_t spinLimitTicks;  // bound of one in-kernel wait, in 100 MHz ticks
   uint32_t* status;         // device status word (HELIX_A2A_STATUS_* bits)
   // combine only

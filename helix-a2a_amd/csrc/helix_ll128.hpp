@@ -219,4 +219,17 @@ HELIX_HD int entries_for_msgs(int msgs, const MsgShape& s) {
   return (msgs + per - 1) / per;
 }
 
+// Units a lane keeps in flight per pass when the largest run of a launch has
+// `runUnits` units: the fewest passes of at most kMaxUnitsInFlight units per
+// lane, then the smallest count that still makes that number of passes (a run
+// of 4.5 units per lane takes one pass of 5, not one of 6 with a wasted slot;
+// one of 10 takes two passes of 5, not 6 + 4).
+constexpr int kMaxUnitsInFlight = 6;
+HELIX_HD int units_in_flight_for_run(long runUnits) {
+  long perLane = (runUnits + kWaveLanes - 1) / kWaveLanes;
+  if (perLane < 1) perLane = 1;
+  long passes = (perLane + kMaxUnitsInFlight - 1) / kMaxUnitsInFlight;
+  return static_cast<int>((perLane + passes - 1) / passes);
+}
+
 }  // namespace helix

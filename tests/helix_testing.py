@@ -58,6 +58,8 @@ class HostModel:
         lib.hm_msg_lines.restype = ctypes.c_int
         lib.hm_unit_first_piece.argtypes = [ctypes.c_int]
         lib.hm_unit_first_piece.restype = ctypes.c_int
+        lib.hm_units_in_flight.argtypes = [ctypes.c_long]
+        lib.hm_units_in_flight.restype = ctypes.c_int
         lib.hm_line_div.argtypes = [ctypes.c_uint32, ctypes.c_int]
         lib.hm_line_div.restype = ctypes.c_uint32
         self.lib = lib

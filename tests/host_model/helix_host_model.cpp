@@ -255,4 +255,7 @@ int hm_line_div_mismatches(int lines) {
   return bad;
 }
 
+// units a lane keeps in flight per pass for a launch whose largest run has `runUnits` units
+int hm_units_in_flight(long runUnits) { return units_in_flight_for_run(runUnits); }
+
 }  // extern "C"

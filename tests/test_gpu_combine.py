@@ -190,6 +190,25 @@ def test_combine_large_messages_many_ranks(hx, ops):
     check(combined, None, oracle_combine(big_o, big_s, 16, 0, ho.bf16_bits_to_f32), "bf16")
 
 
+@pytest.mark.parametrize("cp", [3, 6, 12])
+@pytest.mark.parametrize("tokens", [1, 3, 4, 6, 8, 9, 30])
+def test_combine_every_units_in_flight_variant(hx, ops, cp, tokens):
+    # one channel, 2 heads x 128 + 2 pairs of statistics = 528 bytes = 5 lines = 40 units per message: the run
+    # of `tokens` messages selects the sender program with 1, 2, ... 6 units in flight per lane, and the three
+    # rank counts select the 4-, 8- and 16-lanes-per-slot combine kernels
+    heads, d = 2, 128
+    ws = workspace(hx, cp)
+    g = torch.Generator().manual_seed(100 * cp + tokens)
+    ins_o = [torch.randn(tokens, cp, heads * d, generator=g).to(torch.bfloat16).cuda() for _ in range(cp)]
+    ins_s = [torch.stack((torch.randn(tokens, cp, heads, generator=g) * 2,
+                          1 + torch.rand(tokens, cp, heads, generator=g) * 50), -1)
+             .reshape(tokens, cp, 2 * heads).contiguous().cuda() for _ in range(cp)]
+    combined, lse = hx.alltoall_combine_loopback(ins_o, ins_s, ws, hx.STATS_MAX_SUM, return_lse=True, channel_count=1)
+    torch.cuda.synchronize()
+    assert ops.device_status() == 0
+    check(combined, lse, oracle_combine(ins_o, ins_s, heads, 1, ho.bf16_bits_to_f32), "bf16")
+
+
 def test_combine_while_senders_are_still_writing(hx, ops):
     # few channels: all wavefronts resident at once, the combine half has to wait for its senders
     from helix_a2a.workloads import WORKLOADS, make_inputs

@@ -256,6 +256,26 @@ def test_ragged_shapes(hx, ops, cp, entries, x, s):
         assert outs_o[0].shape == ins_o[0].shape
 
 
+@pytest.mark.parametrize("entries,units_in_flight", [(1, 1), (3, 2), (4, 3), (6, 4), (8, 5), (9, 6), (10, 4), (30, 5)])
+def test_every_units_in_flight_variant(hx, ops, entries, units_in_flight):
+    # one channel, 520-byte messages (5 lines = 40 units): the run of `entries` messages makes the
+    # host pick the kernel instantiation with that many units in flight per lane
+    cp, x = 3, 256
+    ws = get_workspace(hx, cp)
+    g = torch.Generator().manual_seed(4000 + entries)
+    ins_o = [torch.randint(-32768, 32767, (entries, cp, x), generator=g, dtype=torch.int16).view(torch.bfloat16).cuda()
+             for _ in range(cp)]
+    ins_s = [torch.randint(-2**31, 2**31 - 1, (entries, cp, 2), generator=g, dtype=torch.int32).view(torch.float32).cuda()
+             for _ in range(cp)]
+    per_lane = -(-entries * 40 // 64)
+    passes = -(-per_lane // 6)
+    assert -(-per_lane // passes) == units_in_flight          # the case is what its label says
+    outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws, channel_count=1)
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(ins_o, ins_s, outs_o, outs_s)
+
+
 def test_special_values_survive(hx, ops):
     # NaN payloads, infinities, denormals and negative zero are bytes like any other
     cp, entries = 2, 4

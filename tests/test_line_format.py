@@ -107,6 +107,20 @@ def test_line_division_is_exact(host_model):
     assert [host_model.lib.hm_line_div(x, 18) for x in (0, 17, 18, 35, 36, 1007, 1023)] == [0, 0, 1, 1, 2, 55, 56]
 
 
+def test_units_in_flight_rule(host_model):
+    # fewest passes of at most 6 units per lane, then the smallest count that keeps that many passes
+    f = host_model.lib.hm_units_in_flight
+    known = {0: 1, 1: 1, 64: 1, 65: 2, 144: 3, 288: 5, 384: 6, 385: 4, 640: 5, 768: 6, 769: 5, 1104: 6, 8192: 6}
+    assert {u: f(u) for u in known} == known
+    for units in range(1, 8193, 7):
+        k = f(units)
+        per_lane = -(-units // 64)
+        passes = -(-per_lane // 6)
+        assert 1 <= k <= 6
+        assert k * passes >= per_lane          # the run is covered in the minimal number of passes
+        assert (k - 1) * passes < per_lane     # and no smaller count would do
+
+
 def test_repeated_calls_reuse_entries_with_new_steps(host_model):
     cp = 2
     ws = host_model.new_workspace(cp, CU)
