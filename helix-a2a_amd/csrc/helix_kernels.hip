@@ -175,23 +175,33 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
     const uint32_t runUnits = static_cast<uint32_t>(runMsgs) * st.unitsPerMsg;
     for (uint32_t U0 = 0; U0 < runUnits; U0 += kUnitsInFlight * kWaveLanes) {
       u32x2 wa[kUnitsInFlight], wb[kUnitsInFlight];
-      bool needField1 = false;
+      unsigned long long needField1[kUnitsInFlight];  // wave-uniform: lanes of access i that hold statistics pieces
 #pragma unroll
       for (int i = 0; i < kUnitsInFlight; ++i) {
         uint32_t U = U0 + i * kWaveLanes + lane;
         UnitOffsets o = unit_offsets(st, firstMsg, U, U < runUnits);
         wa[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field0, o.a0, 0, kAuxNone);
         wb[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field0, o.b0, 0, kAuxNone);
-        needField1 |= (o.a1 != kOutOfRange) | (o.b1 != kOutOfRange);
+        needField1[i] = __ballot((o.a1 != kOutOfRange) | (o.b1 != kOutOfRange));
       }
-      if (__ballot(needField1) != 0ull) {
+      // Statistics are the last few pieces of a message: only the accesses that
+      // cover the end of a message read the second tensor at all.
+      u32x2 sa[kUnitsInFlight], sb[kUnitsInFlight];
 #pragma unroll
-        for (int i = 0; i < kUnitsInFlight; ++i) {
+      for (int i = 0; i < kUnitsInFlight; ++i) {
+        sa[i] = u32x2{0u, 0u};
+        sb[i] = u32x2{0u, 0u};
+        if (needField1[i] != 0ull) {
           uint32_t U = U0 + i * kWaveLanes + lane;
           UnitOffsets o = unit_offsets(st, firstMsg, U, U < runUnits);
-          wa[i] |= __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.a1, 0, kAuxNone);
-          wb[i] |= __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.b1, 0, kAuxNone);
+          sa[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.a1, 0, kAuxNone);
+          sb[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.b1, 0, kAuxNone);
         }
+      }
+#pragma unroll
+      for (int i = 0; i < kUnitsInFlight; ++i) {
+        wa[i] |= sa[i];
+        wb[i] |= sb[i];
       }
       if (U0 == 0) {
         // open the FIFO entry of this run (csrc/helix_alltoall.cu:377-390)
@@ -287,13 +297,19 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
           // returned -- the units of the lines whose flag carries the step. A unit
           // is never read before its line's flag was seen, whatever the
           // granularity at which the memory system serves a 128-byte line.
+          u32x2 f[kUnitsInFlight];
+#pragma unroll
+          for (int i = 0; i < kUnitsInFlight; ++i) {  // all flag loads first: one round trip, not one per access
+            uint32_t U = U0 + i * kWaveLanes + lane;
+            bool isFlagLane = (U & 7u) == 7u;
+            uint32_t off = (pending[i] && isFlagLane) ? entryOffset + U * kUnitBytes + kPieceBytes : kOutOfRange;
+            f[i] = __builtin_amdgcn_raw_buffer_load_b64(st.fifo, off, 0, kAux);
+          }
 #pragma unroll
           for (int i = 0; i < kUnitsInFlight; ++i) {
             uint32_t U = U0 + i * kWaveLanes + lane;
             bool isFlagLane = (U & 7u) == 7u;
-            uint32_t off = (pending[i] && isFlagLane) ? entryOffset + U * kUnitBytes + kPieceBytes : kOutOfRange;
-            u32x2 f = __builtin_amdgcn_raw_buffer_load_b64(st.fifo, off, 0, kAux);
-            bool ok = !pending[i] || !isFlagLane || (f.x == stepLo && f.y == stepHi);
+            bool ok = !pending[i] || !isFlagLane || (f[i].x == stepLo && f[i].y == stepHi);
             unsigned long long okMask = __ballot(ok);
             landed[i] = pending[i] && ((okMask >> flagLane) & 1ull) != 0ull;
           }
@@ -321,7 +337,6 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
           anyPending |= pending[i];
         }
         if (__ballot(!flagsAgree) != 0ull) runClosed = false;  // not what the token promised: go line by line
-        bool needField1 = false;
 #pragma unroll
         for (int i = 0; i < kUnitsInFlight; ++i) {
           uint32_t U = U0 + i * kWaveLanes + lane;
@@ -330,15 +345,8 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
           u32x2 wb = {v[i].z, v[i].w};
           __builtin_amdgcn_raw_buffer_store_b64(wa, st.field0, o.a0, 0, kAuxNt);
           __builtin_amdgcn_raw_buffer_store_b64(wb, st.field0, o.b0, 0, kAuxNt);
-          needField1 |= (o.a1 != kOutOfRange) | (o.b1 != kOutOfRange);
-        }
-        if (__ballot(needField1) != 0ull) {
-#pragma unroll
-          for (int i = 0; i < kUnitsInFlight; ++i) {
-            uint32_t U = U0 + i * kWaveLanes + lane;
-            UnitOffsets o = unit_offsets(st, firstMsg, U, landed[i]);
-            u32x2 wa = {v[i].x, v[i].y};
-            u32x2 wb = {v[i].z, v[i].w};
+          // statistics sit at the end of a message: few accesses touch the second tensor
+          if (__ballot((o.a1 != kOutOfRange) | (o.b1 != kOutOfRange)) != 0ull) {
             __builtin_amdgcn_raw_buffer_store_b64(wa, st.field1, o.a1, 0, kAuxNt);
             __builtin_amdgcn_raw_buffer_store_b64(wb, st.field1, o.b1, 0, kAuxNt);
           }
