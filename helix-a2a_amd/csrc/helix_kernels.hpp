@@ -36,6 +36,7 @@ struct KernelArgs {
   int rankBegin, rankCount;
   int doSend, doRecv;
   int unitsInFlight;        // units_in_flight_for_run(largest run of the launch), 1..kMaxUnitsInFlight
+  int alignedStores;        // receivers realign payload to 16-byte stores: set when runs take several passes
   uint64_t spinLimitTicks;  // bound of one in-kernel wait, in 100 MHz ticks
   uint32_t* status;         // device status word (HELIX_A2A_STATUS_* bits)
   // combine only

@@ -276,6 +276,31 @@ def test_every_units_in_flight_variant(hx, ops, entries, units_in_flight):
     check_against_oracle(ins_o, ins_s, outs_o, outs_s)
 
 
+@pytest.mark.parametrize("cp,entries,x,s,channels", [
+    (3, 40, 136, 10, 2),    # 312 bytes = 3 lines (odd), 20 messages per stream: two passes of four units
+    (2, 200, 8, 6, 2),      # 40 bytes = one line per message, 100 messages per stream
+    (5, 26, 600, 2, 2),     # 1208 bytes = 11 lines, the pass boundary falls inside a message
+    (4, 12, 1016, 14, 1),   # 2088 bytes = 18 lines with 56 bytes of statistics astride two lines
+    (2, 9, 61432, 2, 1),    # 122872 bytes = 1024 lines: one message per FIFO entry, 22 passes each
+    (16, 64, 264, 2, 4),    # 536 bytes = 5 lines, 16 ranks
+])
+def test_runs_of_several_passes(hx, ops, cp, entries, x, s, channels):
+    # runs longer than one pass go through the kernels whose receivers realign the payload to 16-byte stores
+    ws = get_workspace(hx, cp)
+    g = torch.Generator().manual_seed(cp * 977 + entries)
+    ins_o = [torch.randint(-32768, 32767, (entries, cp, x), generator=g, dtype=torch.int16).view(torch.bfloat16).cuda()
+             for _ in range(cp)]
+    ins_s = [torch.randint(-2**31, 2**31 - 1, (entries, cp, s), generator=g, dtype=torch.int32).view(torch.float32).cuda()
+             for _ in range(cp)]
+    lines = -(-(2 * x + 4 * s) // 120)
+    run_units = min(-(-entries // channels), 1024 // lines) * lines * 8
+    assert run_units > 6 * 64
+    outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws, channel_count=channels)
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(ins_o, ins_s, outs_o, outs_s)
+
+
 def test_special_values_survive(hx, ops):
     # NaN payloads, infinities, denormals and negative zero are bytes like any other
     cp, entries = 2, 4
