@@ -48,6 +48,8 @@ struct Ctx {
   MsgShape sh;
   Extent ws;
   Checker chk;
+  int unitsInFlight;   // per round, by the library's rule
+  bool alignedStores;  // receivers of multi-pass runs store realigned 16-byte pieces
 };
 
 Extent field_extent(const helix_a2a_field_t& f, int entries, int cp) {
@@ -160,27 +162,70 @@ void run_receiver(Ctx& c, int r, int s, int ch) {
       sinfo[1] = step;
     }
     uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
-    for (uint32_t U = 0; U < runUnits; ++U) {
-      const uint8_t* src = fifo + entryOffset + U * kUnitBytes;
-      if (!c.chk.ok(fifoExt, src, 16, "fifo load")) continue;
-      uint64_t words[2];
-      memcpy(words, src, 16);
-      uint64_t flag;  // flag of this lane's line
-      memcpy(&flag, fifo + entryOffset + (U | 7u) * kUnitBytes + 8, 8);
-      if (flag != static_cast<uint64_t>(step)) {
-        if (c.chk.violations++ == 0)
-          snprintf(c.chk.first, sizeof(c.chk.first), "stream %d->%d ch %d unit %u: flag %llx != step %llx", s, r, ch, U,
-                   (unsigned long long)flag, (unsigned long long)step);
-        continue;
+    uint8_t* base0 = const_cast<uint8_t*>(e0.base);
+    uint8_t* base1 = const_cast<uint8_t*>(e1.base);
+    const uint32_t stride0 = p.recv_fields[0].stride_bytes, stride1 = p.recv_fields[1].stride_bytes;
+    const uint32_t np0 = static_cast<uint32_t>(c.sh.np0);
+    // one pass = unitsInFlight accesses of 64 lanes, all loaded before anything is stored
+    const uint32_t passUnits = static_cast<uint32_t>(c.unitsInFlight) * kWaveLanes;
+    for (uint32_t U0 = 0; U0 < runUnits; U0 += passUnits) {
+      uint64_t words[kMaxUnitsInFlight][kWaveLanes][2];
+      bool landed[kMaxUnitsInFlight][kWaveLanes];
+      for (int i = 0; i < c.unitsInFlight; ++i) {
+        for (int lane = 0; lane < kWaveLanes; ++lane) {
+          const uint32_t U = U0 + i * kWaveLanes + lane;
+          landed[i][lane] = false;
+          words[i][lane][0] = words[i][lane][1] = 0;  // what an out-of-range load returns
+          if (U >= runUnits) continue;
+          const uint8_t* src = fifo + entryOffset + U * kUnitBytes;
+          if (!c.chk.ok(fifoExt, src, 16, "fifo load")) continue;
+          memcpy(words[i][lane], src, 16);
+          uint64_t flag;  // flag of this lane's line
+          memcpy(&flag, fifo + entryOffset + (U | 7u) * kUnitBytes + 8, 8);
+          if (flag != static_cast<uint64_t>(step)) {
+            if (c.chk.violations++ == 0)
+              snprintf(c.chk.first, sizeof(c.chk.first), "stream %d->%d ch %d unit %u: flag %llx != step %llx", s, r, ch,
+                       U, (unsigned long long)flag, (unsigned long long)step);
+            continue;
+          }
+          landed[i][lane] = true;
+        }
       }
-      UnitOffsets o = unit_offsets(c, firstRow, rowStep, p.recv_fields[0].stride_bytes, p.recv_fields[1].stride_bytes,
-                                   firstMsg, U);
-      const uint32_t offs0[2] = {o.a0, o.b0}, offs1[2] = {o.a1, o.b1};
-      uint8_t* base0 = const_cast<uint8_t*>(e0.base);
-      uint8_t* base1 = const_cast<uint8_t*>(e1.base);
-      for (int k = 0; k < 2; ++k) {
-        if (offs0[k] != kNone && c.chk.ok(e0, base0 + offs0[k], 8, "recv field 0")) memcpy(base0 + offs0[k], &words[k], 8);
-        if (offs1[k] != kNone && c.chk.ok(e1, base1 + offs1[k], 8, "recv field 1")) memcpy(base1 + offs1[k], &words[k], 8);
+      for (int i = 0; i < c.unitsInFlight; ++i) {
+        for (int lane = 0; lane < kWaveLanes; ++lane) {
+          if (!landed[i][lane]) continue;
+          const uint32_t U = U0 + i * kWaveLanes + lane;
+          UnitOffsets o = unit_offsets(c, firstRow, rowStep, stride0, stride1, firstMsg, U);
+          const uint64_t* w = words[i][lane];
+          if (c.alignedStores) {
+            // the 16 aligned bytes that start at this lane's even piece; second half from the next unit
+            const bool haveNext = lane < kWaveLanes - 1 || i + 1 < c.unitsInFlight;
+            const uint64_t nextFirst = lane < kWaveLanes - 1 ? words[i][lane + 1][0] : (haveNext ? words[i + 1][0][0] : 0);
+            RunUnit d = decode_run_unit(U, static_cast<uint32_t>(c.sh.lines), line_div_magic(c.sh.lines));
+            const uint32_t rowBase = (firstRow + (firstMsg + d.msg) * rowStep) * stride0;
+            const bool odd = (d.piece0 & 1u) != 0;
+            const uint32_t c0 = d.piece0 + (odd ? 1u : 0u);
+            const bool takesNext = odd || d.flag;
+            if (c0 < np0 && !(odd && d.flag) && (!takesNext || haveNext)) {
+              const uint64_t chunk[2] = {odd ? w[1] : w[0], takesNext ? nextFirst : w[1]};
+              uint8_t* dst = base0 + rowBase + c0 * kPieceBytes;
+              if (c.chk.ok(e0, dst, 16, "recv field 0 (16 bytes)")) memcpy(dst, chunk, 16);
+            }
+            const bool alone = d.piece0 < np0 && ((i == c.unitsInFlight - 1 && lane == kWaveLanes - 1 && !odd && d.flag) ||
+                                                  (i == 0 && lane == 0 && odd));
+            if (alone) {
+              uint8_t* dst = base0 + rowBase + d.piece0 * kPieceBytes;
+              if (c.chk.ok(e0, dst, 8, "recv field 0 (lone piece)")) memcpy(dst, &w[0], 8);
+            }
+          } else {
+            const uint32_t offs0[2] = {o.a0, o.b0};
+            for (int k = 0; k < 2; ++k)
+              if (offs0[k] != kNone && c.chk.ok(e0, base0 + offs0[k], 8, "recv field 0")) memcpy(base0 + offs0[k], &w[k], 8);
+          }
+          const uint32_t offs1[2] = {o.a1, o.b1};
+          for (int k = 0; k < 2; ++k)
+            if (offs1[k] != kNone && c.chk.ok(e1, base1 + offs1[k], 8, "recv field 1")) memcpy(base1 + offs1[k], &w[k], 8);
+        }
       }
     }
   }
@@ -221,6 +266,13 @@ int hm_alltoall(const helix_a2a_params_t* per_rank, int cp, int cu_count, int ch
     c.entryBegin = static_cast<int>(begin);
     long end = begin + roundEntries;
     c.entryEnd = end > p0.entry_count ? p0.entry_count : static_cast<int>(end);
+    {  // what launch_exchange derives from the round's largest run (channel 0's first)
+      const int msgs0 = stream_msg_count(c.entryBegin, c.entryEnd, 0, channels);
+      const int perEntry = msgs_per_fifo_entry(c.sh);
+      const long maxRun = static_cast<long>(msgs0 < perEntry ? msgs0 : perEntry) * c.sh.units;
+      c.unitsInFlight = units_in_flight_for_run(maxRun);
+      c.alignedStores = maxRun > static_cast<long>(kMaxUnitsInFlight) * kWaveLanes;
+    }
     if (do_send)
       for (int s = 0; s < cp; ++s)
         for (int ch = 0; ch < channels; ++ch)
