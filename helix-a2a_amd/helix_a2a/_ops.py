@@ -252,7 +252,7 @@ class _LogicalRankGroup:
 
     def __init__(self, cp_size: int) -> None:
         self.cp_size = cp_size
-        self.pending: Dict[int, Tuple[_Params, tuple, torch.cuda.Event]] = {}
+        self.pending: Dict[int, Tuple[_Params, tuple, torch.cuda.Event, torch.cuda.Stream]] = {}
         self.signature: Optional[tuple] = None
 
     def submit(self, rank: int, params: _Params, keep: tuple, signature: tuple) -> None:
@@ -261,22 +261,35 @@ class _LogicalRankGroup:
         if self.pending:
             _require(signature == self.signature, "logical ranks of one group must exchange tensors of one shape and dtype")
         self.signature = signature
-        _check(_lib.helix_a2a_alltoall_send(ctypes.byref(params), 1, _stream_handle()), "alltoall (send half)")
+        stream = torch.cuda.current_stream()
+        _check(_lib.helix_a2a_alltoall_send(ctypes.byref(params), 1, stream.cuda_stream), "alltoall (send half)")
         ev = torch.cuda.Event()
-        ev.record()
-        self.pending[rank] = (params, keep, ev)
+        ev.record(stream)
+        self.pending[rank] = (params, keep, ev, stream)
         if len(self.pending) == self.cp_size:
             self._flush()
 
     def _flush(self) -> None:
+        """Enqueue the receive half of every rank on the last caller's stream.
+
+        That stream first waits for every rank's send half; afterwards the
+        stream of every other rank waits for the receive launch, so each
+        rank's outputs are valid once the stream *it* called on has drained.
+        """
         arr = (_Params * self.cp_size)()
         stream = torch.cuda.current_stream()
         for r in range(self.cp_size):
-            params, _keep, ev = self.pending[r]
+            params, _keep, ev, _rank_stream = self.pending[r]
             arr[r] = params
             stream.wait_event(ev)
         try:
-            _check(_lib.helix_a2a_alltoall_recv(arr, self.cp_size, _stream_handle()), "alltoall (receive half)")
+            _check(_lib.helix_a2a_alltoall_recv(arr, self.cp_size, stream.cuda_stream), "alltoall (receive half)")
+            others = {s.cuda_stream: s for _p, _k, _e, s in self.pending.values() if s.cuda_stream != stream.cuda_stream}
+            if others:
+                done = torch.cuda.Event()
+                done.record(stream)
+                for s in others.values():
+                    s.wait_event(done)
         finally:
             self.pending.clear()
             self.signature = None

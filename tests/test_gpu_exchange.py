@@ -681,3 +681,26 @@ def test_empty_inputs(hx, ops):
     got_o, got_s = hx.alltoall_loopback(o1, s1, ws)
     torch.cuda.synchronize()
     check_against_oracle(o1, s1, got_o, got_s)
+
+
+def test_per_rank_calls_on_separate_streams(hx, ops):
+    # every logical rank calls on a stream of its own and waits for that stream only
+    cp, entries = 4, 96
+    ws = get_workspace(hx, cp)
+    g = torch.Generator().manual_seed(23)
+    ins_o = [torch.randn(entries, cp, 1024, generator=g).to(torch.bfloat16).cuda() for _ in range(cp)]
+    ins_s = [torch.randn(entries, cp, 16, generator=g).cuda() for _ in range(cp)]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(cp)]
+    for _ in range(3):
+        outs = [None] * cp
+        for r in (2, 0, 3, 1):
+            with torch.cuda.stream(streams[r]):
+                outs[r] = hx.alltoall(ins_o[r], ins_s[r], ws, cp_rank=r, cp_size=cp)
+        snap = []
+        for r in range(cp):
+            streams[r].synchronize()          # only the rank's own stream
+            snap.append((outs[r][0].clone(), outs[r][1].clone()))
+        torch.cuda.synchronize()
+        check_against_oracle(ins_o, ins_s, [a for a, _ in snap], [b for _, b in snap])
+    assert_clean(ops)
