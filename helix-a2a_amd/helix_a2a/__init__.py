@@ -154,24 +154,12 @@ def dcp_a2a_lse_reduce(
     directly (the reference path permutes before and after its kernel,
     patches/dcp_alltoall_helix.py:545-593).
     """
-    n = len(cp_attn_out)
-    if n < 1 or len(cp_attn_lse) != n:
-        raise RuntimeError("need one attention output and one LSE tensor per rank")
-    outs, stats = [], []
-    for o, lse in zip(cp_attn_out, cp_attn_lse):
-        if o.dim() != 3 or lse.dim() != 2 or o.shape[:2] != lse.shape or o.size(1) % n != 0:
-            raise RuntimeError("expected cp_attn_out [B, H, D] and cp_attn_lse [B, H] with H divisible by the rank count")
-        b, h, d = o.shape
-        outs.append(o.contiguous().view(b, n, (h // n) * d))
-        lse = lse.contiguous()
-        if not is_lse_base_on_e:
-            lse = lse * 0.6931471805599453  # base-2 LSE -> natural log
-        stats.append(lse.view(b, n, h // n))
-    res = _ops.alltoall_combine_loopback(outs, stats, workspace, STATS_LSE_PACKED, return_lse, channel_count)
-    b, h, d = cp_attn_out[0].shape
+    if not is_lse_base_on_e:
+        cp_attn_lse = [lse * 0.6931471805599453 for lse in cp_attn_lse]  # base-2 LSE -> natural log
+    res = _ops.dcp_reduce(cp_attn_out, cp_attn_lse, workspace, return_lse, channel_count)
     if return_lse:
         combined, lses = res
         if not is_lse_base_on_e:
             lses = [t * 1.4426950408889634 for t in lses]
-        return [c.view(b, h // n, d) for c in combined], lses
-    return [c.view(b, h // n, d) for c in res]
+        return combined, lses
+    return res

@@ -13,6 +13,7 @@ from __future__ import annotations
 
 import ctypes
 import os
+import threading
 from pathlib import Path
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -170,6 +171,7 @@ def initialize_workspace(workspace: torch.Tensor, cp_rank: int, cp_size: int) ->
     row_ptr = workspace.data_ptr() + cp_rank * workspace.stride(0) * 8
     # a reset starts a new epoch: half-finished exchanges of logical ranks on this workspace are void
     _groups.pop((workspace.device.index or 0, workspace.data_ptr(), cp_size), None)
+    _reduce_descriptors.clear()
     with torch.cuda.device(workspace.device):
         _check(_lib.helix_a2a_init_workspace(row_ptr, cp_size, 0, _stream_handle()), "init_workspace")
 
@@ -462,6 +464,98 @@ def alltoall_combine_loopback(partial_o: Sequence[torch.Tensor], softmax_stats: 
                               channel_count: int = 0):
     """One fused exchange + combine of all logical ranks; see :class:`CombinePlan`."""
     return CombinePlan(partial_o, softmax_stats, workspace, stats_mode, return_lse, channel_count).run()
+
+
+class _ReduceDescriptors:
+    """Descriptor arrays of one ``dcp_a2a_lse_reduce`` shape, filled once; a call only swaps data pointers."""
+
+    def __init__(self, cp_size: int, batch: int, heads: int, head_dim: int, dtype: torch.dtype,
+                 workspace: torch.Tensor, channel_count: int) -> None:
+        hp = heads // cp_size
+        self.arr = (_Params * cp_size)()
+        self.out = (_CombineOut * cp_size)()
+        self.dtype_code = 0 if dtype == torch.bfloat16 else 1
+        max_ch = max_channel_count(cp_size)
+        elt = 2
+        for r in range(cp_size):
+            p = self.arr[r]
+            f0, f1 = p.send_fields[0], p.send_fields[1]
+            f0.element_count, f0.element_size, f0.stride_bytes = hp * head_dim, elt, hp * head_dim * elt
+            f1.element_count, f1.element_size, f1.stride_bytes = hp, 4, hp * 4
+            p.entry_count = batch
+            p.workspace = workspace.data_ptr()
+            p.workspace_stride_u64 = workspace.stride(0)
+            p.cp_rank, p.cp_size = r, cp_size
+            p.channel_count, p.max_channel_count = int(channel_count), max_ch
+            self.out[r].lse_out = None
+
+
+_reduce_descriptors: Dict[tuple, _ReduceDescriptors] = {}
+_reduce_lock = threading.Lock()  # the cached arrays are rewritten by every call
+
+
+def dcp_reduce(cp_attn_out: Sequence[torch.Tensor], cp_attn_lse: Sequence[torch.Tensor], workspace: torch.Tensor,
+               return_lse: bool, channel_count: int):
+    """Fused exchange + combine of ``[B, H, D]`` / ``[B, H]`` (natural-log LSE) per rank; see ``helix_a2a.dcp_a2a_lse_reduce``.
+
+    Same kernel call as :class:`CombinePlan` with ``STATS_LSE_PACKED``; the
+    descriptor arrays are kept per shape so that a call in a serving loop costs
+    a few pointer stores and the output allocations.
+    """
+    n = len(cp_attn_out)
+    _require(1 <= n <= MAX_CP_SIZE and len(cp_attn_lse) == n, "need one attention output and one LSE tensor per rank")
+    o0 = cp_attn_out[0]
+    _require(isinstance(o0, torch.Tensor) and o0.dim() == 3, "expected cp_attn_out [B, H, D]")
+    shape, dtype, device = o0.shape, o0.dtype, o0.device
+    b, h, d = shape
+    lse_shape = shape[:2]
+    _require(dtype in (torch.float16, torch.bfloat16), "cp_attn_out must be half or bfloat16")
+    _require(o0.is_cuda, "cp_attn_out must be on the GPU")
+    _require(h % n == 0, "H must be divisible by the rank count")
+    hp = h // n
+    _require(hp % 2 == 0, "H / N must be even (LSE rows are exchanged in 8-byte pieces)")
+    _require(d % 4 == 0 and d >= 32, "head_dim must be a multiple of 4 and >= 32")
+    _check_workspace(workspace, n)
+    _require(workspace.device == device, "all tensors must live on one device")
+    key = (n, b, h, d, dtype, workspace.data_ptr(), workspace.stride(0), int(channel_count), device.index)
+    with _reduce_lock:
+        desc = _reduce_descriptors.get(key)
+        if desc is None:
+            if len(_reduce_descriptors) >= 64:
+                _reduce_descriptors.clear()
+            desc = _reduce_descriptors[key] = _ReduceDescriptors(n, b, h, d, dtype, workspace, channel_count)
+    combined: List[torch.Tensor] = []
+    lses: Optional[List[torch.Tensor]] = [] if return_lse else None
+    keep = []
+    with _reduce_lock, torch.cuda.device(device):
+        for r in range(n):
+            o, lse = cp_attn_out[r], cp_attn_lse[r]
+            _require(o.shape == shape and o.dtype == dtype and o.device == device,
+                     "all ranks must pass cp_attn_out of one shape, dtype and device")
+            _require(lse.shape == lse_shape and lse.dtype == torch.float32 and lse.device == device,
+                     "cp_attn_lse must be float32 [B, H] on the same device")
+            if not o.is_contiguous():
+                o = o.contiguous()
+            if not lse.is_contiguous():
+                lse = lse.contiguous()
+            keep.append((o, lse))
+            c = torch.empty((b, hp, d), dtype=dtype, device=device)
+            combined.append(c)
+            p = desc.arr[r]
+            p.send_fields[0].data = o.data_ptr()
+            p.send_fields[1].data = lse.data_ptr()
+            desc.out[r].combined = c.data_ptr()
+            if return_lse:
+                lo = torch.empty((b, hp), dtype=torch.float32, device=device)
+                lses.append(lo)
+                desc.out[r].lse_out = lo.data_ptr()
+            else:
+                desc.out[r].lse_out = None
+        rc = _lib.helix_a2a_alltoall_combine_loopback(desc.arr, desc.out, n, STATS_LSE_PACKED, desc.dtype_code,
+                                                      _stream_handle())
+    if rc != 0:
+        _raise_last("dcp_a2a_lse_reduce")
+    return (combined, lses) if return_lse else combined
 
 
 def device_status() -> int:

@@ -304,3 +304,43 @@ def test_pipeline_benchmark_formulations_agree(hx, ops):
     res = pb.bench_eager(pb.pipeline_recipe, outs, lses, ws, warmup=1, iters=3)
     assert set(res) == {"total", "copy", "a2a", "combine"}
     assert ops.device_status() == 0
+
+
+def test_dcp_a2a_lse_reduce_argument_checks_and_descriptor_reuse(hx, ops):
+    n, b, h, d = 4, 5, 8, 64
+    ws = workspace(hx, n)
+    g = torch.Generator().manual_seed(5)
+
+    def make(bb=b, hh=h, dd=d, dtype=torch.bfloat16):
+        return ([torch.randn(bb, hh, dd, generator=g).to(dtype).cuda() for _ in range(n)],
+                [torch.randn(bb, hh, generator=g).cuda() for _ in range(n)])
+
+    outs, lses = make()
+    bad = [
+        (outs[:3], lses, "one attention output"),                                   # rank count mismatch
+        ([o.float() for o in outs], lses, "half or bfloat16"),
+        ([o.cpu() for o in outs], lses, "GPU"),
+        (outs, [l.double() for l in lses], "float32"),
+        (outs[:3] + [outs[3][:, :4]], lses, "one shape"),
+        (make(hh=6)[0], make(hh=6)[1], "divisible"),
+        (make(hh=4)[0], make(hh=4)[1], "even"),                                     # one head per rank
+        (make(dd=16)[0], make(dd=16)[1], "head_dim"),
+    ]
+    for o, l, pattern in bad:
+        with pytest.raises(RuntimeError, match=pattern):
+            hx.dcp_a2a_lse_reduce(o, l, ws)
+    # the cached descriptor arrays of a shape serve fresh tensors on every call
+    for _ in range(3):
+        outs, lses = make()
+        got, got_lse = hx.dcp_a2a_lse_reduce(outs, lses, ws, return_lse=True)
+        torch.cuda.synchronize()
+        want, want_lse = ho.lse_combine(np.stack([ho.bf16_bits_to_f32(torch_bits(o)) for o in outs]),
+                                        np.stack([l.cpu().numpy() for l in lses]), dtype=np.float64)
+        for r in range(n):
+            ref = want[:, r * (h // n):(r + 1) * (h // n), :]
+            assert (np.abs(got[r].float().cpu().numpy() - ref) <= ATOL + RTOL * np.abs(ref)).all()
+            assert np.allclose(got_lse[r].cpu().numpy(), want_lse[:, r * (h // n):(r + 1) * (h // n)], atol=1e-4)
+    # an empty batch launches nothing
+    e_o, e_l = make(bb=0)
+    assert all(t.shape == (0, h // n, d) for t in hx.dcp_a2a_lse_reduce(e_o, e_l, ws))
+    assert ops.device_status() == 0
