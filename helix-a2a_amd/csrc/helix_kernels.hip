@@ -12,9 +12,9 @@
 //
 // The messages a stream puts into one FIFO entry form a "run": they follow
 // each other without gaps from line 0 of the entry, so a wavefront walks a
-// run as one flat sequence of 16-byte units, kUnitsInFlight units per lane at
-// a time, regardless of message boundaries. All loads of a chunk are issued
-// before the first store.
+// run as one flat sequence of 16-byte units, in passes of up to six units per
+// lane, regardless of message boundaries. All loads of a pass are issued
+// before its first store.
 //
 // Every global access goes through a buffer descriptor that spans exactly the
 // tensor (or the one FIFO) it belongs to: the hardware returns zero for loads

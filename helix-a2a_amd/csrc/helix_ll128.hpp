@@ -138,39 +138,6 @@ HELIX_HD int stream_msg_count(int entryBegin, int entryEnd, int channel, int run
   return (entryEnd - first + runChannels - 1) / runChannels;
 }
 
-// FIFO-entry cursor shared by sender and receiver: both walk the same
-// sequence of (step, line offset) pairs because both apply this rule to the
-// same message size (csrc/helix_alltoall.cu:377-390,427-436).
-struct FifoCursor {
-  int64_t step;   // head (sender) or tail (receiver) counter value of the open entry
-  int lineBase;   // next free line inside the open entry
-  bool open;      // false until the first message of the call
-};
-
-HELIX_HD FifoCursor make_cursor(int64_t counter) {
-  FifoCursor c;
-  c.step = counter;
-  c.lineBase = kFifoEntryLines;  // forces "open a new entry" on the first message
-  c.open = false;
-  return c;
-}
-
-// Returns true when the message of `lines` lines does not fit and a new entry
-// must be opened (the caller then publishes / back-pressures as its role needs).
-HELIX_HD bool cursor_needs_new_entry(const FifoCursor& c, int lines) {
-  return c.lineBase + lines > kFifoEntryLines;
-}
-// Open the next entry. `closedOne` tells the caller a full entry was finished.
-HELIX_HD void cursor_open_entry(FifoCursor& c, bool* closedOne) {
-  *closedOne = c.open;
-  if (c.open) c.step += 1;
-  c.open = true;
-  c.lineBase = 0;
-}
-HELIX_HD int cursor_entry_index(const FifoCursor& c) {
-  return static_cast<int>(c.step & (kFifoDepth - 1));
-}
-
 // Division of a line index x < 1024 by the lines-per-message count L <= 1024
 // without an integer divide: floor(x / L) == (x * M) >> 20 with
 // M = ceil(2^20 / L). Exact on that range: the excess x * (M - 2^20/L) / 2^20
