@@ -45,7 +45,7 @@ def percentile(sorted_vals, q):
     return sorted_vals[i]
 
 
-def cpu_baseline(w, budget_s: float = 12.0):
+def cpu_baseline(w, algorithmic_bytes: int, budget_s: float = 12.0):
     """Time the CPU restatements on this host for the same workload (bounded sample)."""
     import torch
 
@@ -92,7 +92,7 @@ def cpu_baseline(w, budget_s: float = 12.0):
     model_times.sort()
     m50 = percentile(model_times, 0.5)
     return {
-        "value": w.exchange_bytes / p50 / 1e9,
+        "value": algorithmic_bytes / p50 / 1e9,
         "unit": "GB/s",
         "us_per_call": p50 * 1e6,
         "cores": threads,
@@ -150,7 +150,6 @@ def main() -> int:
         helix_a2a.init_workspace(ws, r, w.cp)
     ins_o, ins_s = make_inputs(w, "cuda")
     entries = w.tokens
-    bytes_exchange, bytes_combine = w.exchange_bytes, w.combine_bytes
     if args.layout == "head":
         if args.combine:
             print("bench.py: --combine is measured on the token layout", file=sys.stderr)
@@ -158,13 +157,16 @@ def main() -> int:
         pairs = [as_head_layout(w, o, s) for o, s in zip(ins_o, ins_s)]
         ins_o, ins_s = [p[0] for p in pairs], [p[1] for p in pairs]
         entries = w.tokens * w.heads_per_rank
-        msg = 2 * w.head_dim + 8
-        bytes_exchange = w.cp * w.cp * entries * (2 * msg + 2 * 128 * (-(-msg // 120)))
     if args.combine:
         plan = _ops.CombinePlan(ins_o, ins_s, ws, _ops.STATS_MAX_SUM, False, args.channels)
     else:
         plan = _ops.LoopbackPlan(ins_o, ins_s, ws, args.channels)
     channels = args.channels or _ops.auto_channel_count(w.cp, entries)
+    # algorithmic bytes: payload read + lines written + lines read + output written, with the lines this
+    # channel count makes (the messages of a run are packed piece by piece, whole lines per run)
+    per_head = args.layout == "head"
+    wire = w.run_wire_bytes(channels, per_head)
+    bytes_per_call = w.combine_bytes(channels) if args.combine else w.exchange_bytes(channels, per_head)
 
     for _ in range(args.warmup):
         plan.run()
@@ -200,7 +202,6 @@ def main() -> int:
     status = _ops.device_status()
     avg_kernel_ms = region_start.elapsed_time(region_end) / args.steps  # launch-to-launch, gaps included
     ms_per_step = wall * 1e3 / args.steps
-    bytes_per_call = bytes_combine if args.combine else bytes_exchange
 
     # distribution of single calls (event pair per call), outside the timed region
     n_dist = min(args.steps, 500)
@@ -271,7 +272,7 @@ def main() -> int:
             "channels": channels,
             "launch": f"HIP graph of {args.graph} calls" if args.graph else "eager, one C call per step",
             "algorithmic_bytes_per_call": bytes_per_call,
-            "payload_bytes": w.payload_bytes, "wire_bytes": w.wire_bytes,
+            "payload_bytes": w.payload_bytes, "wire_bytes": wire,
         },
         "kernel_us_in_timed_region": avg_kernel_ms * 1e3,
         "single_call_us": {
@@ -293,7 +294,7 @@ def main() -> int:
         },
     }
     if not args.no_cpu_baseline and not args.combine and args.layout == "token":
-        result["cpu_baseline"] = cpu_baseline(w)
+        result["cpu_baseline"] = cpu_baseline(w, bytes_per_call)
     print(json.dumps(result))
     return 0 if ok else 1
 

@@ -249,7 +249,7 @@ int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs,
   a.sendBytes1 = static_cast<uint32_t>(rows * a.sendStride1);
   a.recvBytes0 = static_cast<uint32_t>(rows * a.recvStride0);
   a.recvBytes1 = static_cast<uint32_t>(rows * a.recvStride1);
-  a.lineMagic = line_div_magic(sh.lines);
+  a.npMagic = div_magic(static_cast<uint32_t>(sh.np));
   a.rankBegin = p0.cp_rank;
   a.rankCount = count;
   a.spinLimitTicks = g_spinLimitUs.load() * 100ull;
@@ -417,7 +417,7 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, cons
     // wavefronts per (receiver, channel): enough to cover a round's units once, and to fill the device
     int msgs = stream_msg_count(a.entryBegin, a.entryEnd, 0, a.runChannels);
     int perEntry = msgs_per_fifo_entry(plan.shape);
-    long runUnits = static_cast<long>(msgs < perEntry ? msgs : perEntry) * plan.shape.units;
+    long runUnits = run_units(msgs < perEntry ? msgs : perEntry, plan.shape);
     long cover = (runUnits + kWaveLanes - 1) / kWaveLanes;
     long fill = static_cast<long>(plan.cuCount) * 16 / (static_cast<long>(cp_size) * a.runChannels);
     long parts = cover < fill ? cover : fill;

@@ -113,7 +113,7 @@ struct Stream {
   uint32_t stride0, stride1;      // row strides in bytes
   uint32_t firstRow;              // row of the stream's first message of this launch
   uint32_t rowStep;               // rows between consecutive messages of the stream
-  uint32_t np0, np, lines, unitsPerMsg, magic;
+  uint32_t np0, np, npMagic;       // pieces of field 0, of a message, div_magic(np)
   int msgs;                       // messages of the stream in this launch
   int msgsPerEntry;
 };
@@ -122,13 +122,17 @@ __device__ __forceinline__ void setup_stream(Stream& st, const KernelArgs& a, in
   const MsgShape sh = make_msg_shape(a.field0Bytes, a.field1Bytes);
   st.np0 = sh.np0;
   st.np = sh.np;
-  st.lines = sh.lines;
-  st.unitsPerMsg = sh.units;
-  st.magic = a.lineMagic;
+  st.npMagic = a.npMagic;
   st.msgsPerEntry = msgs_per_fifo_entry(sh);
   st.msgs = stream_msg_count(a.entryBegin, a.entryEnd, ch, a.runChannels);
   st.firstRow = static_cast<uint32_t>(a.entryBegin + ch) * a.cpSize + peer;
   st.rowStep = static_cast<uint32_t>(a.runChannels) * a.cpSize;
+}
+
+// 16-byte units of a run of `msgs` messages of this stream's shape
+__device__ __forceinline__ uint32_t stream_run_units(const Stream& st, int msgs) {
+  const uint32_t pieces = static_cast<uint32_t>(msgs) * st.np;
+  return (pieces + kPiecesPerLine - 1) / kPiecesPerLine * kUnitsPerLine;
 }
 
 // Byte offsets of the two payload pieces of run unit U inside the field
@@ -139,19 +143,23 @@ struct UnitOffsets {
   uint32_t a1, b1;  // ... in field 1
 };
 
-__device__ __forceinline__ UnitOffsets unit_offsets(const Stream& st, uint32_t firstMsg, uint32_t U, bool live) {
-  RunUnit d = decode_run_unit(U, st.lines, st.magic);
-  uint32_t row = st.firstRow + (firstMsg + d.msg) * st.rowStep;
-  uint32_t base0 = row * st.stride0;
-  uint32_t base1 = row * st.stride1;
-  uint32_t pa = d.piece0;
-  uint32_t pb = d.piece0 + 1;
-  bool bLive = live && !d.flag;
+// `runMsgs` bounds the run: pieces of later messages are padding of the last line.
+__device__ __forceinline__ UnitOffsets unit_offsets(const Stream& st, uint32_t firstMsg, uint32_t runMsgs, uint32_t U,
+                                                    bool live, RunUnit* decoded = nullptr) {
+  const RunUnit d = decode_run_unit(U, st.np, st.npMagic);
+  const uint32_t rowA = st.firstRow + (firstMsg + d.msgA) * st.rowStep;
+  const uint32_t rowB = d.msgB == d.msgA ? rowA : rowA + st.rowStep;
+  const uint32_t baseA0 = rowA * st.stride0, baseA1 = rowA * st.stride1;
+  const uint32_t baseB0 = rowB * st.stride0, baseB1 = rowB * st.stride1;
+  const bool aLive = live && d.msgA < runMsgs;
+  const bool bLive = live && !d.flag && d.msgB < runMsgs;
+  const uint32_t pa = d.pieceA, pb = d.pieceB;
   UnitOffsets o;
-  o.a0 = (live && pa < st.np0) ? base0 + pa * kPieceBytes : kOutOfRange;
-  o.b0 = (bLive && pb < st.np0) ? base0 + pb * kPieceBytes : kOutOfRange;
-  o.a1 = (live && pa >= st.np0 && pa < st.np) ? base1 + (pa - st.np0) * kPieceBytes : kOutOfRange;
-  o.b1 = (bLive && pb >= st.np0 && pb < st.np) ? base1 + (pb - st.np0) * kPieceBytes : kOutOfRange;
+  o.a0 = (aLive && pa < st.np0) ? baseA0 + pa * kPieceBytes : kOutOfRange;
+  o.b0 = (bLive && pb < st.np0) ? baseB0 + pb * kPieceBytes : kOutOfRange;
+  o.a1 = (aLive && pa >= st.np0) ? baseA1 + (pa - st.np0) * kPieceBytes : kOutOfRange;
+  o.b1 = (bLive && pb >= st.np0) ? baseB1 + (pb - st.np0) * kPieceBytes : kOutOfRange;
+  if (decoded) *decoded = d;
   return o;
 }
 
@@ -178,14 +186,14 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
 
   for (int firstMsg = 0; firstMsg < st.msgs; firstMsg += st.msgsPerEntry) {
     const int runMsgs = min(st.msgsPerEntry, st.msgs - firstMsg);
-    const uint32_t runUnits = static_cast<uint32_t>(runMsgs) * st.unitsPerMsg;
+    const uint32_t runUnits = stream_run_units(st, runMsgs);
     for (uint32_t U0 = 0; U0 < runUnits; U0 += kUnitsInFlight * kWaveLanes) {
       u32x2 wa[kUnitsInFlight], wb[kUnitsInFlight];
       unsigned long long needField1[kUnitsInFlight];  // wave-uniform: lanes of access i that hold statistics pieces
 #pragma unroll
       for (int i = 0; i < kUnitsInFlight; ++i) {
         uint32_t U = U0 + i * kWaveLanes + lane;
-        UnitOffsets o = unit_offsets(st, firstMsg, U, U < runUnits);
+        UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < runUnits);
         wa[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field0, o.a0, 0, kAuxNone);
         wb[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field0, o.b0, 0, kAuxNone);
         needField1[i] = __ballot((o.a1 != kOutOfRange) | (o.b1 != kOutOfRange));
@@ -199,7 +207,7 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
         sb[i] = u32x2{0u, 0u};
         if (needField1[i] != 0ull) {
           uint32_t U = U0 + i * kWaveLanes + lane;
-          UnitOffsets o = unit_offsets(st, firstMsg, U, U < runUnits);
+          UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < runUnits);
           sa[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.a1, 0, kAuxNone);
           sb[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.b1, 0, kAuxNone);
         }
@@ -271,7 +279,7 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
 
   for (int firstMsg = 0; firstMsg < st.msgs; firstMsg += st.msgsPerEntry) {
     const int runMsgs = min(st.msgsPerEntry, st.msgs - firstMsg);
-    const uint32_t runUnits = static_cast<uint32_t>(runMsgs) * st.unitsPerMsg;
+    const uint32_t runUnits = stream_run_units(st, runMsgs);
     if (firstMsg > 0) {
       // every line of the previous entry has been consumed: hand it back to
       // the sender (csrc/helix_alltoall.cu:427-449)
@@ -348,24 +356,27 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
 #pragma unroll
         for (int i = 0; i < kUnitsInFlight; ++i) {
           uint32_t U = U0 + i * kWaveLanes + lane;
-          UnitOffsets o = unit_offsets(st, firstMsg, U, landed[i]);
+          RunUnit d;
+          UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, landed[i], &d);
           u32x2 wa = {v[i].x, v[i].y};
           u32x2 wb = {v[i].z, v[i].w};
           if (store16s) {
-            // A line carries 15 pieces, so on the odd lines of a message a unit's
-            // two pieces sit astride a 16-byte boundary of the row. With the whole
-            // pass in registers every lane stores the aligned 16 bytes that start
-            // at its even piece instead, taking the second half from the next
-            // unit (the next lane; for lane 63 lane 0 of the next access):
-            //   even line:  units 0..6 store their own two pieces, the flag unit
-            //               stores its piece + the first piece of the next line;
-            //   odd line:   units 0..6 store their second piece + the first of
-            //               the next unit, the flag unit stores nothing.
-            // Where the pass ends between the two halves, both are stored alone.
-            // (Costs a dozen vector instructions per unit and halves the store
-            // instructions: measured on MI355X it is 5-6 % faster on runs of
-            // several passes and 2 % slower on single-pass runs, hence a template
-            // parameter the host sets through KernelArgs::alignedStores.)
+            // Messages follow each other piece by piece and a line carries 15 of
+            // them, so the two pieces of a unit sit astride a 16-byte boundary
+            // of the output row about half of the time, and the two 8-byte stores
+            // of an access then each write every other 8 bytes. With the whole
+            // pass in registers every lane stores the aligned 16 bytes ("chunk")
+            // that start at whichever of its words is an even partial_o piece:
+            //   first word even:   both own words, or -- in the flag unit -- the
+            //                      own word + the first word of the next unit;
+            //   second word even:  that word + the first word of the next unit;
+            // the next unit being the next lane (for lane 63, lane 0 of the next
+            // access). An odd first word belongs to the previous unit's chunk.
+            // Where the pass ends between the halves of a chunk, both are stored
+            // alone. (Costs a dozen vector instructions per unit and halves the
+            // store instructions: measured on MI355X it is 5-6 % faster on runs
+            // of several passes and 2 % slower on single-pass runs, hence a
+            // template parameter the host sets through KernelArgs::alignedStores.)
             uint32_t nx = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v[i].x), kDppWaveShl1, 0xF, 0xF, false));
             uint32_t ny = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v[i].y), kDppWaveShl1, 0xF, 0xF, false));
             const bool haveNext = lane < kWaveLanes - 1 || i + 1 < kUnitsInFlight;
@@ -377,20 +388,20 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
                 ny = fy;
               }
             }
-            const RunUnit d = decode_run_unit(U, st.lines, st.magic);
-            const uint32_t base0 = (st.firstRow + (firstMsg + d.msg) * st.rowStep) * st.stride0;
-            const bool odd = (d.piece0 & 1u) != 0u;
-            const uint32_t c0 = d.piece0 + (odd ? 1u : 0u);  // the even piece this lane's 16 bytes start at
-            const bool takesNext = odd || d.flag;
-            const bool store16 = landed[i] && c0 < st.np0 && !(odd && d.flag) && (!takesNext || haveNext);
-            u32x4 chunk = {odd ? v[i].z : v[i].x, odd ? v[i].w : v[i].y, takesNext ? nx : v[i].z, takesNext ? ny : v[i].w};
-            __builtin_amdgcn_raw_buffer_store_b128(chunk, st.field0, store16 ? base0 + c0 * kPieceBytes : kOutOfRange, 0, kAuxNt);
-            // the halves of a pair the pass boundary separates: the last lane's flag unit, the first lane's first piece
-            const bool alone = landed[i] && d.piece0 < st.np0 &&
-                               ((i == kUnitsInFlight - 1 && lane == kWaveLanes - 1 && !odd && d.flag) ||
-                                (i == 0 && lane == 0 && odd));
+            const bool startsAtA = o.a0 != kOutOfRange && (d.pieceA & 1u) == 0u;
+            const bool startsAtB = o.b0 != kOutOfRange && (d.pieceB & 1u) == 0u;
+            const bool takesNext = startsAtB || (startsAtA && d.flag);
+            const bool store16 = (startsAtA || startsAtB) && (!takesNext || haveNext);
+            u32x4 chunk = {startsAtB ? v[i].z : v[i].x, startsAtB ? v[i].w : v[i].y, takesNext ? nx : v[i].z,
+                           takesNext ? ny : v[i].w};
+            __builtin_amdgcn_raw_buffer_store_b128(chunk, st.field0, store16 ? (startsAtB ? o.b0 : o.a0) : kOutOfRange, 0,
+                                                   kAuxNt);
+            // the halves of a chunk the pass boundary separates: the last lane's flag unit, the first lane's first word
+            const bool alone = o.a0 != kOutOfRange &&
+                               ((i == kUnitsInFlight - 1 && lane == kWaveLanes - 1 && startsAtA && d.flag) ||
+                                (i == 0 && lane == 0 && (d.pieceA & 1u) != 0u));
             if ((i == 0 || i == kUnitsInFlight - 1) && __ballot(alone) != 0ull)
-              __builtin_amdgcn_raw_buffer_store_b64(wa, st.field0, alone ? base0 + d.piece0 * kPieceBytes : kOutOfRange, 0, kAuxNt);
+              __builtin_amdgcn_raw_buffer_store_b64(wa, st.field0, alone ? o.a0 : kOutOfRange, 0, kAuxNt);
           } else {
             __builtin_amdgcn_raw_buffer_store_b64(wa, st.field0, o.a0, 0, kAuxNt);
             __builtin_amdgcn_raw_buffer_store_b64(wb, st.field0, o.b0, 0, kAuxNt);
@@ -517,7 +528,7 @@ struct CombineCtx {
 };
 
 struct CombineLds {
-  uint32_t slot[kMaxCombineParts][kCombineSlots][4];          // {first line of the message in the run, head, entry, -}
+  uint32_t slot[kMaxCombineParts][kCombineSlots][4];          // {first run piece of the message, head, entry, -}
   float weight[kMaxCombineParts][kCombineSlots][kMaxCpSize];  // normalised softmax weight per sender
 };
 
@@ -592,7 +603,7 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
 
   for (int firstMsg = 0; firstMsg < st.msgs; firstMsg += st.msgsPerEntry, myStep += 1) {
     const int runMsgs = min(st.msgsPerEntry, st.msgs - firstMsg);
-    const uint32_t runUnits = static_cast<uint32_t>(runMsgs) * st.unitsPerMsg;
+    const uint32_t runUnits = stream_run_units(st, runMsgs);
     cx.stepLo = static_cast<uint32_t>(myStep);
     cx.stepHi = static_cast<uint32_t>(static_cast<uint64_t>(myStep) >> 32);
     {
@@ -614,15 +625,18 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
     for (uint32_t U0 = static_cast<uint32_t>(part) * kWaveLanes; U0 < runUnits;
          U0 += static_cast<uint32_t>(parts) * kWaveLanes) {
       const uint32_t U = U0 + lane;
-      const RunUnit d = decode_run_unit(U, st.lines, st.magic);
+      const RunUnit d = decode_run_unit(U, st.np, st.npMagic);
       const bool live = U < runUnits;
-      const bool dataA = live && d.piece0 < st.np0;
-      const bool dataB = live && !d.flag && d.piece0 + 1 < st.np0;
-      if (__ballot(dataA) == 0ull) continue;  // statistics, padding: nothing to reduce here
-      const uint32_t hA = head_of_piece(d.piece0, a.headMagic);
-      const uint32_t hB = dataB ? head_of_piece(d.piece0 + 1, a.headMagic) : hA;
-      const bool ownB = dataB && hB != hA;  // the second piece starts the next head
-      const uint32_t entry = static_cast<uint32_t>(a.entryBegin + ch) + (firstMsg + d.msg) * a.runChannels;
+      const bool dataA = live && d.msgA < static_cast<uint32_t>(runMsgs) && d.pieceA < st.np0;
+      const bool dataB = live && !d.flag && d.msgB < static_cast<uint32_t>(runMsgs) && d.pieceB < st.np0;
+      if (__ballot(dataA || dataB) == 0ull) continue;  // statistics, padding: nothing to reduce here
+      const uint32_t hA = head_of_piece(d.pieceA, a.headMagic);
+      const uint32_t hB = head_of_piece(d.pieceB, a.headMagic);
+      const uint32_t pairA = d.msgA * static_cast<uint32_t>(a.heads) + hA;
+      const uint32_t pairB = d.msgB * static_cast<uint32_t>(a.heads) + hB;
+      const bool ownB = dataB && (!dataA || pairB != pairA);  // the second piece starts the next head (or message)
+      const uint32_t entryA = static_cast<uint32_t>(a.entryBegin + ch) + (firstMsg + d.msgA) * a.runChannels;
+      const uint32_t entryB = static_cast<uint32_t>(a.entryBegin + ch) + (firstMsg + d.msgB) * a.runChannels;
 
       // Up to eight senders: their unit loads go out before the weights are
       // worked out -- they do not depend on them, and the two round trips
@@ -646,8 +660,7 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
       if (kLoadUnitsEarly) load_units(0);
 
       // ---- slots: one per distinct (message, head) the lanes of this access touch, in lane order
-      const uint32_t pairA = d.msg * static_cast<uint32_t>(a.heads) + hA;
-      const uint32_t lastPair = dataA ? (ownB ? pairA + 1u : pairA) : 0xFFFFFFFFu;
+      const uint32_t lastPair = dataB ? pairB : (dataA ? pairA : 0xFFFFFFFFu);
       const uint32_t prevPair = shuffle_from(lastPair, lane == 0 ? 0 : lane - 1);
       const bool newA = dataA && (lane == 0 || prevPair != pairA);
       const unsigned long long startsA = __ballot(newA), startsB = __ballot(ownB);
@@ -659,14 +672,14 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
         return;
       }
       if (newA) {
-        lds.slot[part][slotA][0] = d.msg * st.lines;
+        lds.slot[part][slotA][0] = d.msgA * st.np;
         lds.slot[part][slotA][1] = hA;
-        lds.slot[part][slotA][2] = entry;
+        lds.slot[part][slotA][2] = entryA;
       }
       if (ownB) {
-        lds.slot[part][slotB][0] = d.msg * st.lines;
+        lds.slot[part][slotB][0] = d.msgB * st.np;
         lds.slot[part][slotB][1] = hB;
-        lds.slot[part][slotB][2] = entry;
+        lds.slot[part][slotB][2] = entryB;
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
@@ -678,14 +691,14 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
         const int q = lane % kLanesPerSlot;
         const bool serving = slot < slotCount && q < a.cpSize;
         const int slotSafe = slot < kCombineSlots ? slot : 0;
-        const uint32_t msgLine0 = lds.slot[part][slotSafe][0];
+        const uint32_t msgPiece0 = lds.slot[part][slotSafe][0];
         const uint32_t h = lds.slot[part][slotSafe][1];
         const uint32_t slotEntry = lds.slot[part][slotSafe][2];
-        const uint32_t ps = st.np0 + (a.statsMode == 2 ? h >> 1 : h);  // statistics piece of head h
-        const uint32_t ls = ps / kPiecesPerLine;
-        const uint32_t word = ps - ls * kPiecesPerLine;
+        const uint32_t gs = msgPiece0 + st.np0 + (a.statsMode == 2 ? h >> 1 : h);  // run piece that holds head h's statistics
+        const uint32_t ls = gs / kPiecesPerLine;
+        const uint32_t word = gs - ls * kPiecesPerLine;
         const uint32_t qStepLo = shuffle_from(cx.stepLo, q < a.cpSize ? q : 0);
-        const uint32_t off = entry_base(cx, q, qStepLo) + (msgLine0 + ls) * kLineBytes + word * kPieceBytes;
+        const uint32_t off = entry_base(cx, q, qStepLo) + ls * kLineBytes + word * kPieceBytes;
         const u32x2 sv = __builtin_amdgcn_raw_buffer_load_b64(cx.fifos, serving ? off : kOutOfRange, 0, kAuxSc1);
         const float lse = serving ? lse_of_stats(sv.x, sv.y, a.statsMode, h) : -INFINITY;
         float m = lse;
@@ -709,7 +722,7 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
 
       // ---- the unit of every sender, weighted
       const float* wA = lds.weight[part][dataA ? slotA : 0];
-      const float* wB = lds.weight[part][dataA ? slotB : 0];
+      const float* wB = lds.weight[part][dataB ? slotB : 0];
       float accA[4] = {0.0f, 0.0f, 0.0f, 0.0f};
       float accB[4] = {0.0f, 0.0f, 0.0f, 0.0f};
       uint32_t flagMismatch = 0u;
@@ -742,11 +755,10 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
         raise_status(a.status, kStatusInternal, lane);
         return;
       }
-      const uint32_t rowByte = entry * (st.np0 * kPieceBytes);
       __builtin_amdgcn_raw_buffer_store_b64(narrow_piece<kDtype>(accA), outRsrc,
-                                            dataA ? rowByte + d.piece0 * kPieceBytes : kOutOfRange, 0, kAuxNone);
+                                            dataA ? (entryA * st.np0 + d.pieceA) * kPieceBytes : kOutOfRange, 0, kAuxNone);
       __builtin_amdgcn_raw_buffer_store_b64(narrow_piece<kDtype>(accB), outRsrc,
-                                            dataB ? rowByte + (d.piece0 + 1) * kPieceBytes : kOutOfRange, 0, kAuxNone);
+                                            dataB ? (entryB * st.np0 + d.pieceB) * kPieceBytes : kOutOfRange, 0, kAuxNone);
       __builtin_amdgcn_wave_barrier();  // the tables are rewritten by the next access
     }
   }
@@ -794,7 +806,7 @@ static KernelArgs with_units_in_flight(KernelArgs a) {
   const MsgShape sh = make_msg_shape(a.field0Bytes, a.field1Bytes);
   const int msgs = stream_msg_count(a.entryBegin, a.entryEnd, 0, a.runChannels);
   const int perEntry = msgs_per_fifo_entry(sh);
-  const long runUnits = static_cast<long>(msgs < perEntry ? msgs : perEntry) * sh.units;
+  const long runUnits = run_units(msgs < perEntry ? msgs : perEntry, sh);
   a.unitsInFlight = units_in_flight_for_run(runUnits);
   a.alignedStores = runUnits > static_cast<long>(kMaxUnitsInFlight) * kWaveLanes ? 1 : 0;
   return a;

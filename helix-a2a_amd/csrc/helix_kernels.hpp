@@ -32,7 +32,7 @@ struct KernelArgs {
   int recvStride0, recvStride1;
   uint32_t sendBytes0, sendBytes1;  // extent of each tensor (< 2 GiB), the range of its buffer descriptor
   uint32_t recvBytes0, recvBytes1;
-  uint32_t lineMagic;               // line_div_magic(lines per message)
+  uint32_t npMagic;                 // div_magic(pieces per message)
   int rankBegin, rankCount;
   int doSend, doRecv;
   int unitsInFlight;        // units_in_flight_for_run(largest run of the launch), 1..kMaxUnitsInFlight

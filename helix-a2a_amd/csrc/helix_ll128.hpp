@@ -8,7 +8,7 @@
 // line and displaces payload words into tail blocks, csrc/ll128_proto.cuh:73-139):
 //
 //   one line  = 128 bytes = 16 words of 8 bytes
-//   words 0..14  payload pieces 15*l .. 15*l+14 of the message (l = line index)
+//   words 0..14  payload pieces 15*l .. 15*l+14 of the run (l = line index)
 //   word  15     flag = the FIFO step counter under which the line was written
 //
 //   one unit  = 16 bytes = words (2u, 2u+1) of a line, u = 0..7. A lane moves
@@ -16,8 +16,11 @@
 //   wavefront covers 8 lines (1 KiB), and the lane with u == 7 carries
 //   {payload piece 15*l+14, flag} in a single 16-byte store.
 //
-// A message is field 0 followed by field 1, cut into 8-byte pieces; the last
-// line is zero padded.
+// A message is field 0 followed by field 1, cut into 8-byte pieces. A run is
+// the messages a stream puts into one FIFO entry, piece after piece without
+// gaps: message j of the run is run pieces j*np .. (j+1)*np - 1, wherever the
+// line boundaries fall (a 264-byte message is 33 pieces = 2.2 lines, not 3).
+// Only the last line of a run is zero padded.
 //
 // Workspace geometry (one row per rank, unchanged from the reference so that
 // workspace_size and the init pattern stay drop-in,
@@ -102,8 +105,7 @@ HELIX_HD uint64_t receiver_info_offset(int cpSize, int maxCh, int sender, int ch
 struct MsgShape {
   int np0;    // 8-byte pieces of field 0
   int np;     // pieces of field 0 + field 1
-  int lines;  // LL128 lines on the wire
-  int units;  // 16-byte units on the wire = 8 * lines
+  int lines;  // LL128 lines of a message on its own (what must fit one FIFO entry)
 };
 
 HELIX_HD MsgShape make_msg_shape(int field0Bytes, int field1Bytes) {
@@ -111,23 +113,18 @@ HELIX_HD MsgShape make_msg_shape(int field0Bytes, int field1Bytes) {
   s.np0 = field0Bytes / kPieceBytes;
   s.np = s.np0 + field1Bytes / kPieceBytes;
   s.lines = (s.np + kPiecesPerLine - 1) / kPiecesPerLine;
-  s.units = s.lines * kUnitsPerLine;
   return s;
 }
 
-HELIX_HD int msgs_per_fifo_entry(const MsgShape& s) { return kFifoEntryLines / s.lines; }
+// messages one FIFO entry (1024 lines = 15 360 pieces) holds
+HELIX_HD int msgs_per_fifo_entry(const MsgShape& s) { return kFifoEntryLines * kPiecesPerLine / s.np; }
+// lines and 16-byte units of a run of `msgs` messages
+HELIX_HD int run_lines(int msgs, const MsgShape& s) { return (msgs * s.np + kPiecesPerLine - 1) / kPiecesPerLine; }
+HELIX_HD int run_units(int msgs, const MsgShape& s) { return run_lines(msgs, s) * kUnitsPerLine; }
 
-// first payload piece carried by unit g (= line*8 + u) of a message; the
-// second word of the unit is piece+1, or the flag when (g & 7) == 7.
+// first payload piece carried by unit g (= line*8 + u) of a run; the second
+// word of the unit is piece+1, or the flag when (g & 7) == 7.
 HELIX_HD int unit_first_piece(int g) { return (g >> 3) * kPiecesPerLine + 2 * (g & 7); }
-HELIX_HD bool unit_has_flag(int g) { return (g & 7) == 7; }
-
-// byte offset of unit g of a message that starts at line `lineBase` of FIFO
-// entry `entry` (0..3), relative to the FIFO base.
-HELIX_HD uint32_t fifo_unit_offset(int entry, int lineBase, int g) {
-  return static_cast<uint32_t>(entry) * kFifoEntryBytes +
-         static_cast<uint32_t>(lineBase) * kLineBytes + static_cast<uint32_t>(g) * kUnitBytes;
-}
 
 // ---- per-stream schedule ------------------------------------------------------
 // Entries e = entryBegin + channel, + runChannels, ... < entryEnd belong to the
@@ -138,46 +135,42 @@ HELIX_HD int stream_msg_count(int entryBegin, int entryEnd, int channel, int run
   return (entryEnd - first + runChannels - 1) / runChannels;
 }
 
-// Division of a line index x < 1024 by the lines-per-message count L <= 1024
-// without an integer divide: floor(x / L) == (x * M) >> 20 with
-// M = ceil(2^20 / L). Exact on that range: the excess x * (M - 2^20/L) / 2^20
-// stays below 2^-10 <= 1/L (and is zero for L = 1024).
-constexpr int kLineDivShift = 20;
-HELIX_HD uint32_t line_div_magic(int lines) {
-  return static_cast<uint32_t>(((1u << kLineDivShift) + lines - 1) / lines);
+// floor(p / d) for p < 2^16 and 1 <= d < 2^16 without an integer divide: a
+// multiply-high by M = floor(2^32 / d) + 1. Exact on that range (the excess
+// p * (M - 2^32/d) / 2^32 is below 2^-16 <= 1/d); d == 1 is the identity and
+// uses magic 0. Run pieces (< 15 360) are divided by the pieces per message
+// with it, pieces of a message by the pieces per head.
+HELIX_HD uint32_t div_magic(uint32_t d) { return d <= 1 ? 0u : static_cast<uint32_t>((1ull << 32) / d) + 1u; }
+HELIX_HD uint32_t div_by_magic(uint32_t p, uint32_t magic) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return magic == 0u ? p : __umulhi(p, magic);
+#else
+  return magic == 0u ? p : static_cast<uint32_t>((static_cast<uint64_t>(p) * magic) >> 32);
+#endif
 }
-HELIX_HD uint32_t line_div(uint32_t x, uint32_t magic) { return (x * magic) >> kLineDivShift; }
 
-// Where unit U of a run lives. A run is the sequence of messages a stream
-// puts into one FIFO entry; it starts at line 0 of the entry and its messages
-// follow each other without gaps, so unit U sits at byte U*16 of the entry.
+// Where unit U of a run lives: the message and the piece inside that message
+// of each of its two words. Unit U sits at byte U*16 of the FIFO entry.
 struct RunUnit {
-  uint32_t msg;     // message index inside the run
-  uint32_t piece0;  // first payload piece of the unit inside its message
-  bool flag;        // second word of the unit is the flag word
+  uint32_t msgA, pieceA;  // first word
+  uint32_t msgB, pieceB;  // second word (the next piece of the run; may start the next message)
+  bool flag;              // ... unless it is the line's flag word
 };
-HELIX_HD RunUnit decode_run_unit(uint32_t U, uint32_t lines, uint32_t magic) {
+HELIX_HD RunUnit decode_run_unit(uint32_t U, uint32_t np, uint32_t npMagic) {
   RunUnit d;
-  uint32_t x = U >> 3;
-  uint32_t u = U & 7u;
-  d.msg = line_div(x, magic);
-  uint32_t line = x - d.msg * lines;
-  d.piece0 = line * kPiecesPerLine + 2u * u;
-  d.flag = u == 7u;
+  const uint32_t g = (U >> 3) * kPiecesPerLine + 2u * (U & 7u);
+  d.msgA = div_by_magic(g, npMagic);
+  d.pieceA = g - d.msgA * np;
+  const bool wraps = d.pieceA + 1u == np;
+  d.msgB = d.msgA + (wraps ? 1u : 0u);
+  d.pieceB = wraps ? 0u : d.pieceA + 1u;
+  d.flag = (U & 7u) == 7u;
   return d;
 }
 
-// Head index of payload piece p when a head spans `piecesPerHead` pieces
-// (head_dim * 2 bytes / 8): floor(p / piecesPerHead) as a multiply-high by
-// M = floor(2^32 / piecesPerHead) + 1. Exact for p < 2^16 and
-// 2 <= piecesPerHead < 2^16 (the excess p * (M - 2^32/d) / 2^32 is below
-// 2^-16 <= 1/d); piecesPerHead == 1 is the identity and uses magic 0.
-HELIX_HD uint32_t head_div_magic(uint32_t piecesPerHead) {
-  return piecesPerHead <= 1 ? 0u : static_cast<uint32_t>((1ull << 32) / piecesPerHead) + 1u;
-}
-HELIX_HD uint32_t head_of_piece(uint32_t p, uint32_t magic) {
-  return magic == 0u ? p : static_cast<uint32_t>((static_cast<uint64_t>(p) * magic) >> 32);
-}
+// Head index of payload piece p when a head spans `piecesPerHead` pieces (head_dim * 2 bytes / 8).
+HELIX_HD uint32_t head_div_magic(uint32_t piecesPerHead) { return div_magic(piecesPerHead); }
+HELIX_HD uint32_t head_of_piece(uint32_t p, uint32_t magic) { return div_by_magic(p, magic); }
 
 // Number of FIFO entries a stream of `msgs` messages consumes in one call.
 HELIX_HD int entries_for_msgs(int msgs, const MsgShape& s) {

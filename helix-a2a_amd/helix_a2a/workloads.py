@@ -46,19 +46,42 @@ class Workload:
 
     @property
     def wire_bytes(self) -> int:
-        """W: bytes of whole LL128 lines (120 payload bytes each) for the same."""
+        """W with every message in whole LL128 lines of its own (120 payload bytes each): the upper bound."""
         lines = -(-(self.field0_bytes + self.field1_bytes) // 120)
         return self.cp * self.cp * self.tokens * 128 * lines
 
-    @property
-    def exchange_bytes(self) -> int:
-        """payload read + FIFO write + FIFO read + output write."""
-        return 2 * self.payload_bytes + 2 * self.wire_bytes
+    def run_wire_bytes(self, channels: int, per_head: bool = False) -> int:
+        """W as this build writes it: the messages of a run packed piece by piece, whole lines per run."""
+        if per_head:
+            return wire_bytes(self.tokens * self.heads_per_rank, 2 * self.head_dim, 8, self.cp, channels)
+        return wire_bytes(self.tokens, self.field0_bytes, self.field1_bytes, self.cp, channels)
 
-    @property
-    def combine_bytes(self) -> int:
+    def exchange_bytes(self, channels: int, per_head: bool = False) -> int:
+        """payload read + FIFO write + FIFO read + output write."""
+        return 2 * self.payload_bytes + 2 * self.run_wire_bytes(channels, per_head)
+
+    def combine_bytes(self, channels: int) -> int:
         """as above with the output write replaced by the combined [T, H/cp, D] tensor."""
-        return self.payload_bytes + 2 * self.wire_bytes + self.cp * self.tokens * self.heads_per_rank * self.head_dim * 2
+        return (self.payload_bytes + 2 * self.run_wire_bytes(channels)
+                + self.cp * self.tokens * self.heads_per_rank * self.head_dim * 2)
+
+
+def wire_bytes(entries: int, field0_bytes: int, field1_bytes: int, cp: int, channels: int) -> int:
+    """Bytes of LL128 lines one call writes into the FIFOs (and reads back), over all cp * cp pairs.
+
+    A stream (pair, channel) carries the entries ``channel, channel + channels, ...``; the messages it puts into
+    one 1024-line FIFO entry form a run, stored piece after piece (8 bytes), 15 pieces + the flag word per line.
+    """
+    pieces = (field0_bytes + field1_bytes) // 8
+    per_entry = 1024 * 15 // pieces
+    lines = 0
+    for ch in range(min(channels, entries)):
+        msgs = len(range(ch, entries, channels))
+        while msgs > 0:
+            run = min(msgs, per_entry)
+            lines += -(-run * pieces // 15)
+            msgs -= run
+    return cp * cp * lines * 128
 
 
 WORKLOADS: Dict[str, Workload] = {

@@ -60,8 +60,14 @@ class HostModel:
         lib.hm_unit_first_piece.restype = ctypes.c_int
         lib.hm_units_in_flight.argtypes = [ctypes.c_long]
         lib.hm_units_in_flight.restype = ctypes.c_int
-        lib.hm_line_div.argtypes = [ctypes.c_uint32, ctypes.c_int]
-        lib.hm_line_div.restype = ctypes.c_uint32
+        lib.hm_div.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
+        lib.hm_div.restype = ctypes.c_uint32
+        lib.hm_div_mismatches.argtypes = [ctypes.c_uint32]
+        lib.hm_div_mismatches.restype = ctypes.c_int
+        lib.hm_run_lines.argtypes = [ctypes.c_int] * 3
+        lib.hm_run_lines.restype = ctypes.c_int
+        lib.hm_msgs_per_entry.argtypes = [ctypes.c_int] * 2
+        lib.hm_msgs_per_entry.restype = ctypes.c_int
         self.lib = lib
 
     @staticmethod

@@ -65,18 +65,20 @@ struct UnitOffsets {
 };
 
 UnitOffsets unit_offsets(const Ctx& c, uint32_t firstRow, uint32_t rowStep, uint32_t stride0, uint32_t stride1,
-                         uint32_t firstMsg, uint32_t U) {
-  RunUnit d = decode_run_unit(U, static_cast<uint32_t>(c.sh.lines), line_div_magic(c.sh.lines));
-  uint32_t row = firstRow + (firstMsg + d.msg) * rowStep;
-  uint32_t base0 = row * stride0, base1 = row * stride1;
-  uint32_t np0 = static_cast<uint32_t>(c.sh.np0), np = static_cast<uint32_t>(c.sh.np);
-  uint32_t pa = d.piece0, pb = d.piece0 + 1;
+                         uint32_t firstMsg, uint32_t runMsgs, uint32_t U, RunUnit* decoded = nullptr) {
+  const uint32_t np0 = static_cast<uint32_t>(c.sh.np0), np = static_cast<uint32_t>(c.sh.np);
+  RunUnit d = decode_run_unit(U, np, div_magic(np));
+  uint32_t rowA = firstRow + (firstMsg + d.msgA) * rowStep;
+  uint32_t rowB = firstRow + (firstMsg + d.msgB) * rowStep;
+  const bool aLive = d.msgA < runMsgs;
+  const bool bLive = !d.flag && d.msgB < runMsgs;
   UnitOffsets o;
   o.flag = d.flag;
-  o.a0 = pa < np0 ? base0 + pa * kPieceBytes : kNone;
-  o.b0 = (!d.flag && pb < np0) ? base0 + pb * kPieceBytes : kNone;
-  o.a1 = (pa >= np0 && pa < np) ? base1 + (pa - np0) * kPieceBytes : kNone;
-  o.b1 = (!d.flag && pb >= np0 && pb < np) ? base1 + (pb - np0) * kPieceBytes : kNone;
+  o.a0 = (aLive && d.pieceA < np0) ? rowA * stride0 + d.pieceA * kPieceBytes : kNone;
+  o.b0 = (bLive && d.pieceB < np0) ? rowB * stride0 + d.pieceB * kPieceBytes : kNone;
+  o.a1 = (aLive && d.pieceA >= np0) ? rowA * stride1 + (d.pieceA - np0) * kPieceBytes : kNone;
+  o.b1 = (bLive && d.pieceB >= np0) ? rowB * stride1 + (d.pieceB - np0) * kPieceBytes : kNone;
+  if (decoded) *decoded = d;
   return o;
 }
 
@@ -101,7 +103,7 @@ void run_sender(Ctx& c, int s, int r, int ch) {
   int64_t step = info[0];
   for (int firstMsg = 0; firstMsg < msgs; firstMsg += perEntry) {
     int runMsgs = perEntry < msgs - firstMsg ? perEntry : msgs - firstMsg;
-    uint32_t runUnits = static_cast<uint32_t>(runMsgs) * c.sh.units;
+    uint32_t runUnits = static_cast<uint32_t>(run_units(runMsgs, c.sh));
     if (firstMsg > 0) {
       step += 1;
       info[0] = step;
@@ -116,7 +118,7 @@ void run_sender(Ctx& c, int s, int r, int ch) {
     uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
     for (uint32_t U = 0; U < runUnits; ++U) {  // every lane of every wave access
       UnitOffsets o = unit_offsets(c, firstRow, rowStep, p.send_fields[0].stride_bytes, p.send_fields[1].stride_bytes,
-                                   firstMsg, U);
+                                   firstMsg, runMsgs, U);
       uint64_t words[2] = {0, 0};
       const uint32_t offs0[2] = {o.a0, o.b0}, offs1[2] = {o.a1, o.b1};
       for (int k = 0; k < 2; ++k) {
@@ -155,7 +157,7 @@ void run_receiver(Ctx& c, int r, int s, int ch) {
   int64_t step = info[1];
   for (int firstMsg = 0; firstMsg < msgs; firstMsg += perEntry) {
     int runMsgs = perEntry < msgs - firstMsg ? perEntry : msgs - firstMsg;
-    uint32_t runUnits = static_cast<uint32_t>(runMsgs) * c.sh.units;
+    uint32_t runUnits = static_cast<uint32_t>(run_units(runMsgs, c.sh));
     if (firstMsg > 0) {
       step += 1;
       info[1] = step;
@@ -165,7 +167,6 @@ void run_receiver(Ctx& c, int r, int s, int ch) {
     uint8_t* base0 = const_cast<uint8_t*>(e0.base);
     uint8_t* base1 = const_cast<uint8_t*>(e1.base);
     const uint32_t stride0 = p.recv_fields[0].stride_bytes, stride1 = p.recv_fields[1].stride_bytes;
-    const uint32_t np0 = static_cast<uint32_t>(c.sh.np0);
     // one pass = unitsInFlight accesses of 64 lanes, all loaded before anything is stored
     const uint32_t passUnits = static_cast<uint32_t>(c.unitsInFlight) * kWaveLanes;
     for (uint32_t U0 = 0; U0 < runUnits; U0 += passUnits) {
@@ -195,26 +196,25 @@ void run_receiver(Ctx& c, int r, int s, int ch) {
         for (int lane = 0; lane < kWaveLanes; ++lane) {
           if (!landed[i][lane]) continue;
           const uint32_t U = U0 + i * kWaveLanes + lane;
-          UnitOffsets o = unit_offsets(c, firstRow, rowStep, stride0, stride1, firstMsg, U);
+          RunUnit d;
+          UnitOffsets o = unit_offsets(c, firstRow, rowStep, stride0, stride1, firstMsg, runMsgs, U, &d);
           const uint64_t* w = words[i][lane];
           if (c.alignedStores) {
-            // the 16 aligned bytes that start at this lane's even piece; second half from the next unit
+            // the aligned 16 bytes that start at whichever word is an even partial_o piece; second half from the next unit
             const bool haveNext = lane < kWaveLanes - 1 || i + 1 < c.unitsInFlight;
             const uint64_t nextFirst = lane < kWaveLanes - 1 ? words[i][lane + 1][0] : (haveNext ? words[i + 1][0][0] : 0);
-            RunUnit d = decode_run_unit(U, static_cast<uint32_t>(c.sh.lines), line_div_magic(c.sh.lines));
-            const uint32_t rowBase = (firstRow + (firstMsg + d.msg) * rowStep) * stride0;
-            const bool odd = (d.piece0 & 1u) != 0;
-            const uint32_t c0 = d.piece0 + (odd ? 1u : 0u);
-            const bool takesNext = odd || d.flag;
-            if (c0 < np0 && !(odd && d.flag) && (!takesNext || haveNext)) {
-              const uint64_t chunk[2] = {odd ? w[1] : w[0], takesNext ? nextFirst : w[1]};
-              uint8_t* dst = base0 + rowBase + c0 * kPieceBytes;
+            const bool startsAtA = o.a0 != kNone && (d.pieceA & 1u) == 0;
+            const bool startsAtB = o.b0 != kNone && (d.pieceB & 1u) == 0;
+            const bool takesNext = startsAtB || (startsAtA && d.flag);
+            if ((startsAtA || startsAtB) && (!takesNext || haveNext)) {
+              const uint64_t chunk[2] = {startsAtB ? w[1] : w[0], takesNext ? nextFirst : w[1]};
+              uint8_t* dst = base0 + (startsAtB ? o.b0 : o.a0);
               if (c.chk.ok(e0, dst, 16, "recv field 0 (16 bytes)")) memcpy(dst, chunk, 16);
             }
-            const bool alone = d.piece0 < np0 && ((i == c.unitsInFlight - 1 && lane == kWaveLanes - 1 && !odd && d.flag) ||
-                                                  (i == 0 && lane == 0 && odd));
+            const bool alone = o.a0 != kNone && ((i == c.unitsInFlight - 1 && lane == kWaveLanes - 1 && startsAtA && d.flag) ||
+                                                 (i == 0 && lane == 0 && (d.pieceA & 1u) != 0));
             if (alone) {
-              uint8_t* dst = base0 + rowBase + d.piece0 * kPieceBytes;
+              uint8_t* dst = base0 + o.a0;
               if (c.chk.ok(e0, dst, 8, "recv field 0 (lone piece)")) memcpy(dst, &w[0], 8);
             }
           } else {
@@ -269,7 +269,7 @@ int hm_alltoall(const helix_a2a_params_t* per_rank, int cp, int cu_count, int ch
     {  // what launch_exchange derives from the round's largest run (channel 0's first)
       const int msgs0 = stream_msg_count(c.entryBegin, c.entryEnd, 0, channels);
       const int perEntry = msgs_per_fifo_entry(c.sh);
-      const long maxRun = static_cast<long>(msgs0 < perEntry ? msgs0 : perEntry) * c.sh.units;
+      const long maxRun = run_units(msgs0 < perEntry ? msgs0 : perEntry, c.sh);
       c.unitsInFlight = units_in_flight_for_run(maxRun);
       c.alignedStores = maxRun > static_cast<long>(kMaxUnitsInFlight) * kWaveLanes;
     }
@@ -297,16 +297,19 @@ uint64_t hm_receiver_info_offset(int cp, int max_ch, int sender, int channel) {
 }
 int hm_msg_lines(int f0, int f1) { return make_msg_shape(f0, f1).lines; }
 int hm_unit_first_piece(int g) { return unit_first_piece(g); }
-// floor(x / lines) the way the kernels compute it
-uint32_t hm_line_div(uint32_t x, int lines) { return line_div(x, line_div_magic(lines)); }
-// number of line indices x of a FIFO entry for which that differs from x / lines
-int hm_line_div_mismatches(int lines) {
+// floor(g / d) the way the kernels compute it
+uint32_t hm_div(uint32_t g, uint32_t d) { return div_by_magic(g, div_magic(d)); }
+// number of run piece indices g of a FIFO entry for which that differs from g / d
+int hm_div_mismatches(uint32_t d) {
   int bad = 0;
-  for (uint32_t x = 0; x < static_cast<uint32_t>(kFifoEntryLines); ++x)
-    bad += line_div(x, line_div_magic(lines)) != x / static_cast<uint32_t>(lines);
+  const uint32_t magic = div_magic(d);
+  for (uint32_t g = 0; g < static_cast<uint32_t>(kFifoEntryLines * kPiecesPerLine) + 16u; ++g)
+    bad += div_by_magic(g, magic) != g / d;
   return bad;
 }
-
+// lines of a run of `msgs` messages and messages per FIFO entry for a message of the two field sizes
+int hm_run_lines(int msgs, int field0_bytes, int field1_bytes) { return run_lines(msgs, make_msg_shape(field0_bytes, field1_bytes)); }
+int hm_msgs_per_entry(int field0_bytes, int field1_bytes) { return msgs_per_fifo_entry(make_msg_shape(field0_bytes, field1_bytes)); }
 // units a lane keeps in flight per pass for a launch whose largest run has `runUnits` units
 int hm_units_in_flight(long runUnits) { return units_in_flight_for_run(runUnits); }
 

@@ -256,10 +256,11 @@ def test_ragged_shapes(hx, ops, cp, entries, x, s):
         assert outs_o[0].shape == ins_o[0].shape
 
 
-@pytest.mark.parametrize("entries,units_in_flight", [(1, 1), (3, 2), (4, 3), (6, 4), (8, 5), (9, 6), (10, 4), (30, 5)])
+@pytest.mark.parametrize("entries,units_in_flight", [(1, 1), (3, 2), (5, 3), (7, 4), (9, 5), (11, 6), (12, 4), (33, 6)])
 def test_every_units_in_flight_variant(hx, ops, entries, units_in_flight):
-    # one channel, 520-byte messages (5 lines = 40 units): the run of `entries` messages makes the
-    # host pick the kernel instantiation with that many units in flight per lane
+    # one channel, 520-byte messages (65 pieces): the run of `entries` messages, packed piece by piece into
+    # ceil(65 * entries / 15) lines of 8 units, makes the host pick the kernel instantiation with that many
+    # units in flight per lane
     cp, x = 3, 256
     ws = get_workspace(hx, cp)
     g = torch.Generator().manual_seed(4000 + entries)
@@ -267,7 +268,7 @@ def test_every_units_in_flight_variant(hx, ops, entries, units_in_flight):
              for _ in range(cp)]
     ins_s = [torch.randint(-2**31, 2**31 - 1, (entries, cp, 2), generator=g, dtype=torch.int32).view(torch.float32).cuda()
              for _ in range(cp)]
-    per_lane = -(-entries * 40 // 64)
+    per_lane = -(-(-(-entries * 65 // 15) * 8) // 64)
     passes = -(-per_lane // 6)
     assert -(-per_lane // passes) == units_in_flight          # the case is what its label says
     outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws, channel_count=1)
@@ -277,12 +278,13 @@ def test_every_units_in_flight_variant(hx, ops, entries, units_in_flight):
 
 
 @pytest.mark.parametrize("cp,entries,x,s,channels", [
-    (3, 40, 136, 10, 2),    # 312 bytes = 3 lines (odd), 20 messages per stream: two passes of four units
-    (2, 200, 8, 6, 2),      # 40 bytes = one line per message, 100 messages per stream
-    (5, 26, 600, 2, 2),     # 1208 bytes = 11 lines, the pass boundary falls inside a message
-    (4, 12, 1016, 14, 1),   # 2088 bytes = 18 lines with 56 bytes of statistics astride two lines
-    (2, 9, 61432, 2, 1),    # 122872 bytes = 1024 lines: one message per FIFO entry, 22 passes each
-    (16, 64, 264, 2, 4),    # 536 bytes = 5 lines, 16 ranks
+    (3, 40, 136, 10, 2),    # 312 bytes = 39 pieces (odd), 20 messages per stream: two passes
+    (2, 400, 8, 6, 2),      # 40 bytes = 5 pieces: three messages per line, 200 per stream
+    (5, 26, 600, 2, 2),     # 1208 bytes = 151 pieces, the pass boundary falls inside a message
+    (4, 12, 1016, 14, 1),   # 2088 bytes = 261 pieces with 56 bytes of statistics astride two lines
+    (2, 9, 61432, 2, 1),    # 122872 bytes = 15 360 pieces: one message per FIFO entry, 22 passes each
+    (16, 64, 264, 2, 4),    # 536 bytes = 67 pieces, 16 ranks
+    (8, 2048, 128, 2, 128), # the benchmark shape passed per head: 264 bytes = 33 pieces, 16 per stream
 ])
 def test_runs_of_several_passes(hx, ops, cp, entries, x, s, channels):
     # runs longer than one pass go through the kernels whose receivers realign the payload to 16-byte stores
@@ -292,9 +294,9 @@ def test_runs_of_several_passes(hx, ops, cp, entries, x, s, channels):
              for _ in range(cp)]
     ins_s = [torch.randint(-2**31, 2**31 - 1, (entries, cp, s), generator=g, dtype=torch.int32).view(torch.float32).cuda()
              for _ in range(cp)]
-    lines = -(-(2 * x + 4 * s) // 120)
-    run_units = min(-(-entries // channels), 1024 // lines) * lines * 8
-    assert run_units > 6 * 64
+    pieces = (2 * x + 4 * s) // 8
+    run_units = -(-min(-(-entries // channels), 15360 // pieces) * pieces // 15) * 8
+    assert run_units > 6 * 64 or entries == 2048
     outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws, channel_count=channels)
     torch.cuda.synchronize()
     assert_clean(ops)
@@ -516,8 +518,8 @@ def test_receive_without_send_times_out_cleanly(hx, ops):
 
 
 def test_send_capacity_is_checked_for_split_phases(hx, ops):
-    # 2-line messages on one channel: 2048 fit the four FIFO entries; a send-only launch of more is refused
-    cp, entries = 2, 2049
+    # 17-piece messages on one channel: 4 x 903 fit the four FIFO entries; a send-only launch of more is refused
+    cp, entries = 2, 3613
     ws = get_workspace(hx, cp)
     o = torch.zeros(entries, cp, 64, dtype=torch.bfloat16, device="cuda")
     s = torch.zeros(entries, cp, 2, device="cuda")
@@ -532,9 +534,9 @@ def test_send_capacity_is_checked_for_split_phases(hx, ops):
 
 @pytest.mark.parametrize("single_round", [False, True])
 def test_traffic_beyond_fifo_capacity(hx, ops, single_round):
-    # 5000 two-line messages per stream on one channel = 10 FIFO entries. Default: three stream-ordered
+    # 9000 messages of 17 pieces per stream on one channel = 10 FIFO entries. Default: three stream-ordered
     # rounds. single_round: one launch, senders wait in-kernel until receivers release entries.
-    cp, entries = 2, 5000
+    cp, entries = 2, 9000
     ws = get_workspace(hx, cp, fresh=True)
     g = torch.Generator().manual_seed(9)
     ins_o = [torch.randint(-32768, 32767, (entries, cp, 64), generator=g, dtype=torch.int16).view(torch.bfloat16).cuda()

@@ -107,11 +107,52 @@ def test_unit_to_piece_map_covers_every_piece_once(host_model):
         assert seen == list(range(15 * lines))
 
 
-def test_line_division_is_exact(host_model):
-    # the multiply-shift that replaces x / lines must be exact for every line index of a FIFO entry
-    for lines in range(1, 1025):
-        assert host_model.lib.hm_line_div_mismatches(lines) == 0, lines
-    assert [host_model.lib.hm_line_div(x, 18) for x in (0, 17, 18, 35, 36, 1007, 1023)] == [0, 0, 1, 1, 2, 55, 56]
+def test_piece_division_is_exact(host_model):
+    # the multiply-high that replaces g / np must be exact for every run piece of a FIFO entry (g < 15 360)
+    # and every message size that fits one (3 <= np <= 15 360); every np up to 2048, then a sample
+    sizes = list(range(1, 2049)) + list(range(2049, 15361, 97)) + [15359, 15360]
+    for d in sizes:
+        assert host_model.lib.hm_div_mismatches(d) == 0, d
+    assert [host_model.lib.hm_div(g, 33) for g in (0, 32, 33, 65, 66, 15359)] == [0, 0, 1, 1, 2, 465]
+
+
+def test_messages_of_a_run_are_packed_piece_by_piece(host_model):
+    # per-head layout of the benchmark shape: 264-byte messages = 33 pieces = 2.2 lines each. Five of them
+    # are 165 pieces = exactly 11 lines, where one message per three lines would take 15.
+    cp, entries, x, s = 2, 5, 128, 2
+    assert host_model.lib.hm_msg_lines(2 * x, 4 * s) == 3
+    assert host_model.lib.hm_run_lines(5, 2 * x, 4 * s) == 11
+    assert host_model.lib.hm_run_lines(16, 2 * x, 4 * s) == 36
+    assert host_model.lib.hm_msgs_per_entry(2 * x, 4 * s) == 15360 // 33
+    assert host_model.lib.hm_msgs_per_entry(2048, 64) == 58          # 264 pieces
+    assert host_model.lib.hm_msgs_per_entry(122872, 8) == 1          # 15 360 pieces: the largest message
+    ins_o, ins_s = random_inputs(cp, entries, x, s, seed=2)
+    ws = host_model.new_workspace(cp, CU)
+    _, _, rc, msg = host_model.alltoall(ins_o, ins_s, ws, CU, 1, send=True, recv=False)
+    assert rc == 0, msg
+    max_ch = host_model.max_channel_count(cp, CU)
+    for sender in range(cp):
+        for receiver in range(cp):
+            off = host_model.lib.hm_fifo_offset(sender, 0, max_ch)
+            fifo = ws[receiver].view(np.uint64)[off // 8: (off + FIFO_BYTES) // 8]
+            lines = fifo[: 11 * 16].reshape(11, 16)
+            run = np.concatenate([np.concatenate([ins_o[sender][e, receiver].view(np.uint64),
+                                                  ins_s[sender][e, receiver].view(np.uint64)]) for e in range(entries)])
+            assert run.size == 165
+            assert (lines[:, :15].reshape(-1) == run).all()          # message after message, no gaps
+            assert (lines[:, 15] == 0).all()                         # every line carries the step
+            assert (fifo[11 * 16:] == np.uint64(0xFFFFFFFFFFFFFFFF)).all()
+    # six messages: 198 pieces = 13.2 lines -> 14 lines, the last one zero padded
+    ins_o, ins_s = random_inputs(cp, 6, x, s, seed=3)
+    ws = host_model.new_workspace(cp, CU)
+    out_o, out_s, rc, msg = host_model.alltoall(ins_o, ins_s, ws, CU, 1)
+    assert rc == 0, msg
+    fifo = ws[1].view(np.uint64)[: FIFO_BYTES // 8]                  # sender 0 -> receiver 1
+    last = fifo[13 * 16: 14 * 16]
+    assert (last[3:15] == 0).all() and last[15] == 0 and (fifo[14 * 16:] == np.uint64(0xFFFFFFFFFFFFFFFF)).all()
+    want_o, want_s = ho.exchange_closed_form(ins_o), ho.exchange_closed_form(ins_s)
+    for r in range(cp):
+        assert np.array_equal(out_o[r], want_o[r]) and np.array_equal(out_s[r], want_s[r])
 
 
 def test_units_in_flight_rule(host_model):
@@ -148,15 +189,15 @@ def test_repeated_calls_reuse_entries_with_new_steps(host_model):
 
 
 def test_rounds_when_traffic_exceeds_the_fifo(host_model):
-    # 2-line messages, one channel: 512 messages per entry, 2048 per round; 5000 entries need 3 rounds
-    cp, entries = 2, 5000
+    # 17-piece messages, one channel: 903 messages per entry, 3612 per round; 9000 entries need 3 rounds
+    cp, entries = 2, 9000
     ins_o, ins_s = random_inputs(cp, entries, 64, 2, seed=7)
     out_o, out_s, ws = _exchange(host_model, ins_o, ins_s, channels=1)
     want_o, want_s = ho.exchange_closed_form(ins_o), ho.exchange_closed_form(ins_s)
     for r in range(cp):
         assert (out_o[r] == want_o[r]).all() and (out_s[r] == want_s[r]).all()
     so = host_model.lib.hm_sender_info_offset(cp, host_model.max_channel_count(cp, CU), 0, 0)
-    assert ws[0][so // 8] == 4 + 4 + 2  # entries consumed: 2048 + 2048 + 904 messages
+    assert ws[0][so // 8] == 4 + 4 + 2  # entries consumed: 3612 + 3612 + 1776 messages
 
 
 def test_receiver_rejects_stale_lines(host_model):
