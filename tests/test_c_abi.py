@@ -190,3 +190,18 @@ def test_combine_argument_validation_without_a_device(ops):
     assert lib.helix_a2a_alltoall_combine_loopback(arr, out, 4, 0, 5, None) == 1
     assert "dtype" in lib.helix_a2a_last_error().decode()
     assert lib.helix_a2a_alltoall_combine_loopback(arr, None, 4, 0, 0, None) == 1
+
+
+def test_header_is_c_and_a_c_host_can_call_the_library(ops, tmp_path):
+    # include/helix_a2a.h compiled as C99 with -pedantic; the program exercises sizes and validation (no device)
+    import subprocess
+
+    src = ROOT / "tests" / "c_abi" / "c_abi_smoke.c"
+    exe = tmp_path / "c_abi_smoke"
+    libdir = Path(ops.library_path()).parent
+    cmd = ["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", f"-I{ROOT / 'include'}", str(src), "-o", str(exe),
+           f"-L{libdir}", "-lhelix_a2a", f"-Wl,-rpath,{libdir}"]
+    build = subprocess.run(cmd, capture_output=True, text=True)
+    assert build.returncode == 0, build.stdout + build.stderr
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert run.returncode == 0 and "c_abi_smoke ok" in run.stdout, run.stdout + run.stderr
