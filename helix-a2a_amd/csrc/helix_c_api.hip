@@ -380,6 +380,9 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, cons
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "unknown stats_mode %d", stats_mode);
   if (dtype != HELIX_A2A_DTYPE_BF16 && dtype != HELIX_A2A_DTYPE_FP16)
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "unknown dtype %d", dtype);
+  if (cp_size > kMaxCombineCpSize)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "the fused combine serves cp_size <= %d, got %d", kMaxCombineCpSize,
+                cp_size);
   Plan plan;
   int rc = build_plan(per_rank, cp_size, false, &plan);
   if (rc) return rc;

@@ -529,7 +529,7 @@ struct CombineCtx {
 
 struct CombineLds {
   uint32_t slot[kMaxCombineParts][kCombineSlots][4];          // {first run piece of the message, head, entry, -}
-  float weight[kMaxCombineParts][kCombineSlots][kMaxCpSize];  // normalised softmax weight per sender
+  float weight[kMaxCombineParts][kCombineSlots][kMaxCombineCpSize];  // normalised softmax weight per sender
 };
 
 __device__ __forceinline__ uint32_t shuffle_from(uint32_t v, int srcLane) {

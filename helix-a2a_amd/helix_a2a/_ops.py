@@ -19,7 +19,8 @@ from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
-MAX_CP_SIZE = 16
+MAX_CP_SIZE = 32
+MAX_COMBINE_CP_SIZE = 16
 
 STATS_LSE = 0          # stats pairs: (natural-log LSE, unused)
 STATS_MAX_SUM = 1      # stats pairs: (running max, running sum)
@@ -412,8 +413,8 @@ class CombinePlan:
                  workspace: torch.Tensor, stats_mode: int = STATS_MAX_SUM, return_lse: bool = False,
                  channel_count: int = 0) -> None:
         cp_size = len(partial_o)
-        _require(1 <= cp_size <= MAX_CP_SIZE and len(softmax_stats) == cp_size,
-                 "need one partial_o and one softmax_stats tensor per rank")
+        _require(1 <= cp_size <= MAX_COMBINE_CP_SIZE and len(softmax_stats) == cp_size,
+                 f"need one partial_o and one softmax_stats tensor per rank, at most {MAX_COMBINE_CP_SIZE} ranks")
         _require(stats_mode in (STATS_LSE, STATS_MAX_SUM, STATS_LSE_PACKED),
                  "stats_mode must be STATS_LSE, STATS_MAX_SUM or STATS_LSE_PACKED")
         _check_workspace(workspace, cp_size)
@@ -503,7 +504,8 @@ def dcp_reduce(cp_attn_out: Sequence[torch.Tensor], cp_attn_lse: Sequence[torch.
     a few pointer stores and the output allocations.
     """
     n = len(cp_attn_out)
-    _require(1 <= n <= MAX_CP_SIZE and len(cp_attn_lse) == n, "need one attention output and one LSE tensor per rank")
+    _require(1 <= n <= MAX_COMBINE_CP_SIZE and len(cp_attn_lse) == n,
+             f"need one attention output and one LSE tensor per rank, at most {MAX_COMBINE_CP_SIZE} ranks")
     o0 = cp_attn_out[0]
     _require(isinstance(o0, torch.Tensor) and o0.dim() == 3, "expected cp_attn_out [B, H, D]")
     shape, dtype, device = o0.shape, o0.dtype, o0.device

@@ -26,7 +26,8 @@ int main(void) {
   CHECK(helix_a2a_workspace_size_per_rank(2, 256) == 134348800LL);
   CHECK(helix_a2a_auto_channel_count(8, 256, 256) == 128);
   CHECK(helix_a2a_auto_channel_count(8, 5, 256) == 5);
-  CHECK(helix_a2a_max_channel_count(17, 256) < 0);
+  CHECK(helix_a2a_max_channel_count(32, 256) == 32);
+  CHECK(helix_a2a_max_channel_count(33, 256) < 0);
   CHECK(strstr(helix_a2a_last_error(), "cp_size") != NULL);
 
   memset(&p, 0, sizeof(p));

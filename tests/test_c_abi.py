@@ -77,7 +77,7 @@ def test_auto_channel_count(ops):
 
 
 def test_bad_arguments_raise_runtime_error(ops):
-    for bad_cp in (0, -1, 17):
+    for bad_cp in (0, -1, 33):
         with pytest.raises(RuntimeError, match="cp_size"):
             ops.get_workspace_size_per_rank(bad_cp, 256)
     with pytest.raises(RuntimeError):
@@ -143,7 +143,7 @@ def test_descriptor_validation_without_a_device(ops):
     send = lib.helix_a2a_alltoall_send
     cases = [
         (dict(cp=0), "cp_size"),
-        (dict(cp=17), "cp_size"),
+        (dict(cp=33), "cp_size"),
         (dict(entries=-1), "entry_count"),
         (dict(rank=4), "cp_rank"),
         (dict(x=100), "multiple of 16 bytes"),          # 200-byte partial_o rows

@@ -158,6 +158,18 @@ def test_combine_4d_inputs_and_plan_replay(hx, ops):
     check(combined, None, want, "bf16")
 
 
+def test_combine_serves_at_most_sixteen_ranks(hx, ops):
+    cp = 17
+    ws = torch.zeros(cp, 8, dtype=torch.int64, device="cuda")  # never reached: the rank count is checked first
+    o = [torch.zeros(1, cp, 64, dtype=torch.bfloat16, device="cuda") for _ in range(cp)]
+    s = [torch.zeros(1, cp, 2, device="cuda") for _ in range(cp)]
+    with pytest.raises(RuntimeError, match="at most 16 ranks"):
+        hx.alltoall_combine_loopback(o, s, ws, hx.STATS_LSE)
+    with pytest.raises(RuntimeError, match="at most 16 ranks"):
+        hx.dcp_a2a_lse_reduce([torch.zeros(1, 34, 32, dtype=torch.bfloat16, device="cuda")] * cp,
+                              [torch.zeros(1, 34, device="cuda")] * cp, ws)
+
+
 def test_combine_rejects_bad_shapes(hx, ops):
     cp = 2
     ws = workspace(hx, cp)

@@ -234,6 +234,8 @@ def test_channel_count_limits(hx, ops):
     (2, 4, 61440, 2),   # 122888 bytes: 1025 lines, more than a FIFO entry holds -> rejected
     (1, 9, 64, 2),      # a single rank talking to itself
     (16, 2, 64, 2),
+    (24, 5, 200, 4),    # more than sixteen ranks: three workgroup columns of eight in the reference's terms
+    (32, 40, 128, 2),   # the largest rank count of an exchange (16 GiB of workspace)
     (4, 0, 64, 2),      # nothing to send
 ])
 def test_ragged_shapes(hx, ops, cp, entries, x, s):

@@ -39,6 +39,8 @@ def _exchange(host_model, ins_o, ins_s, channels, cu=CU, ws=None):
     (4, 12, 1016, 14, 1),  # 2088 bytes = 18 lines with 56 bytes of statistics astride two lines
     (2, 3, 61432, 2, 1),   # 122872 bytes = 1024 lines: one message per FIFO entry
     (16, 64, 264, 2, 2),   # 536 bytes = 5 lines, 16 ranks
+    (32, 3, 64, 2, 1),     # the largest rank count of an exchange
+    (24, 7, 200, 4, 1),
 ])
 def test_host_model_matches_oracle(host_model, cp, entries, x, s, channels):
     ins_o, ins_s = random_inputs(cp, entries, x, s, seed=cp + entries + x)
