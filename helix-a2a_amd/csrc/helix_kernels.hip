@@ -516,7 +516,7 @@ __device__ __forceinline__ uint32_t narrow1<1>(float v) {
 // sideways -- lane j serves slot j / G and sender j % G, loads that sender's
 // statistics of that head, and a softmax over the G lanes of a slot gives
 // the weight -- and the weights go back through LDS to the lanes that own
-// units of the head. (G = 4, 8 or 16 lanes per slot for cpSize <= 4, 8, 16.)
+// units of the head. (G = 4, 8, 16 or 32 lanes per slot for cpSize <= 4, 8, 16, 32.)
 // The `parts` wavefronts of a workgroup split the units of a run.
 constexpr int kCombineSlots = 32;  // distinct (message, head) pairs one wave access may touch
 
@@ -527,9 +527,10 @@ struct CombineCtx {
   uint32_t stepLo, stepHi;       // lane q: step counter of sender q's stream
 };
 
+template <int kLanesPerSlot>
 struct CombineLds {
   uint32_t slot[kMaxCombineParts][kCombineSlots][4];          // {first run piece of the message, head, entry, -}
-  float weight[kMaxCombineParts][kCombineSlots][kMaxCombineCpSize];  // normalised softmax weight per sender
+  float weight[kMaxCombineParts][kCombineSlots][kLanesPerSlot];  // normalised softmax weight per sender
 };
 
 __device__ __forceinline__ uint32_t shuffle_from(uint32_t v, int srcLane) {
@@ -567,7 +568,7 @@ __device__ __forceinline__ u32x2 narrow_piece(const float (&acc)[4]) {
 
 template <int kDtype, int kLanesPerSlot>
 __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r, int ch, int part, int parts,
-                                                     int lane, CombineLds& lds) {
+                                                     int lane, CombineLds<kLanesPerSlot>& lds) {
   constexpr int kSlotsPerPass = kWaveLanes / kLanesPerSlot;
   Stream st;
   setup_stream(st, a, 0, ch);
@@ -769,7 +770,7 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
 // rest receive and combine, one workgroup per (receiver, channel).
 template <int kDtype, int kLanesPerSlot>
 __global__ __launch_bounds__(kMaxCombineParts * kWaveLanes) HELIX_WAVES_PER_SIMD void helix_combine_kernel(KernelArgs a) {
-  __shared__ CombineLds lds;
+  __shared__ CombineLds<kLanesPerSlot> lds;
   const int parts = static_cast<int>(blockDim.x) / kWaveLanes;
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWaveLanes);
   const int lane = static_cast<int>(threadIdx.x) % kWaveLanes;
@@ -851,17 +852,19 @@ hipError_t launch_combine(const KernelArgs& args, int parts, hipStream_t stream)
   if (parts > kMaxCombineParts) parts = kMaxCombineParts;
   const int blocks = (senderStreams + parts - 1) / parts + a.rankCount * a.runChannels;
   dim3 block(static_cast<unsigned>(parts * kWaveLanes));
-  // lanes per slot of the sideways pass: the smallest of 4, 8, 16 that holds every sender
-  const int g = a.cpSize <= 4 ? 4 : a.cpSize <= 8 ? 8 : 16;
+  // lanes per slot of the sideways pass: the smallest of 4, 8, 16, 32 that holds every sender
+  const int g = a.cpSize <= 4 ? 4 : a.cpSize <= 8 ? 8 : a.cpSize <= 16 ? 16 : 32;
 #define HELIX_LAUNCH_COMBINE(DT, G) hipLaunchKernelGGL((helix_combine_kernel<DT, G>), dim3(blocks), block, 0, stream, a)
   if (a.dtype == 1) {
     if (g == 4) HELIX_LAUNCH_COMBINE(1, 4);
     else if (g == 8) HELIX_LAUNCH_COMBINE(1, 8);
-    else HELIX_LAUNCH_COMBINE(1, 16);
+    else if (g == 16) HELIX_LAUNCH_COMBINE(1, 16);
+    else HELIX_LAUNCH_COMBINE(1, 32);
   } else {
     if (g == 4) HELIX_LAUNCH_COMBINE(0, 4);
     else if (g == 8) HELIX_LAUNCH_COMBINE(0, 8);
-    else HELIX_LAUNCH_COMBINE(0, 16);
+    else if (g == 16) HELIX_LAUNCH_COMBINE(0, 16);
+    else HELIX_LAUNCH_COMBINE(0, 32);
   }
 #undef HELIX_LAUNCH_COMBINE
   return hipGetLastError();

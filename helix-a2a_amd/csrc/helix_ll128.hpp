@@ -46,7 +46,7 @@
 namespace helix {
 
 constexpr int kMaxCpSize = 32;         // ranks of one exchange (size of the kernel argument block)
-constexpr int kMaxCombineCpSize = 16;  // ranks of one fused combine (lanes per slot of its sideways pass)
+constexpr int kMaxCombineCpSize = 32;  // ranks of one fused combine (lanes per slot of its sideways pass)
 
 // ---- line format ---------------------------------------------------------
 constexpr int kPieceBytes = 8;

@@ -20,7 +20,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import torch
 
 MAX_CP_SIZE = 32
-MAX_COMBINE_CP_SIZE = 16
+MAX_COMBINE_CP_SIZE = 32
 
 STATS_LSE = 0          # stats pairs: (natural-log LSE, unused)
 STATS_MAX_SUM = 1      # stats pairs: (running max, running sum)

@@ -35,7 +35,7 @@ extern "C" {
 #endif
 
 #define HELIX_A2A_MAX_CP_SIZE 32
-#define HELIX_A2A_MAX_COMBINE_CP_SIZE 16 /* helix_a2a_alltoall_combine_loopback */
+#define HELIX_A2A_MAX_COMBINE_CP_SIZE 32 /* helix_a2a_alltoall_combine_loopback */
 
 /* error codes */
 #define HELIX_A2A_OK 0

@@ -158,16 +158,16 @@ def test_combine_4d_inputs_and_plan_replay(hx, ops):
     check(combined, None, want, "bf16")
 
 
-def test_combine_serves_at_most_sixteen_ranks(hx, ops):
-    cp = 17
+def test_combine_serves_at_most_thirty_two_ranks(hx, ops):
+    cp = 33
     ws = torch.zeros(cp, 8, dtype=torch.int64, device="cuda")  # never reached: the rank count is checked first
     o = [torch.zeros(1, cp, 64, dtype=torch.bfloat16, device="cuda") for _ in range(cp)]
     s = [torch.zeros(1, cp, 2, device="cuda") for _ in range(cp)]
-    with pytest.raises(RuntimeError, match="at most 16 ranks"):
+    with pytest.raises(RuntimeError, match="at most 32 ranks"):
         hx.alltoall_combine_loopback(o, s, ws, hx.STATS_LSE)
-    with pytest.raises(RuntimeError, match="at most 16 ranks"):
-        hx.dcp_a2a_lse_reduce([torch.zeros(1, 34, 32, dtype=torch.bfloat16, device="cuda")] * cp,
-                              [torch.zeros(1, 34, device="cuda")] * cp, ws)
+    with pytest.raises(RuntimeError, match="at most 32 ranks"):
+        hx.dcp_a2a_lse_reduce([torch.zeros(1, 66, 32, dtype=torch.bfloat16, device="cuda")] * cp,
+                              [torch.zeros(1, 66, device="cuda")] * cp, ws)
 
 
 def test_combine_rejects_bad_shapes(hx, ops):
@@ -202,12 +202,12 @@ def test_combine_large_messages_many_ranks(hx, ops):
     check(combined, None, oracle_combine(big_o, big_s, 16, 0, ho.bf16_bits_to_f32), "bf16")
 
 
-@pytest.mark.parametrize("cp", [3, 6, 12])
+@pytest.mark.parametrize("cp", [3, 6, 12, 24])
 @pytest.mark.parametrize("tokens", [1, 3, 5, 7, 9, 11, 33])
 def test_combine_every_units_in_flight_variant(hx, ops, cp, tokens):
     # one channel, 2 heads x 128 + 2 pairs of statistics = 528 bytes = 66 pieces = 4.4 lines per message: the run
-    # of `tokens` messages selects the sender program with 1, 2, ... 6 units in flight per lane, and the three
-    # rank counts select the 4-, 8- and 16-lanes-per-slot combine kernels
+    # of `tokens` messages selects the sender program with 1, 2, ... 6 units in flight per lane, and the four
+    # rank counts select the 4-, 8-, 16- and 32-lanes-per-slot combine kernels
     heads, d = 2, 128
     ws = workspace(hx, cp)
     g = torch.Generator().manual_seed(100 * cp + tokens)
@@ -219,6 +219,24 @@ def test_combine_every_units_in_flight_variant(hx, ops, cp, tokens):
     torch.cuda.synchronize()
     assert ops.device_status() == 0
     check(combined, lse, oracle_combine(ins_o, ins_s, heads, 1, ho.bf16_bits_to_f32), "bf16")
+
+
+def test_combine_thirty_two_ranks(hx, ops):
+    # the largest rank count: 32 senders per (message, head), two slots per sideways pass
+    cp, tokens, heads, d = 32, 20, 2, 64
+    ws = workspace(hx, cp)
+    g = torch.Generator().manual_seed(32)
+    ins_o = [torch.randn(tokens, cp, heads * d, generator=g).to(torch.bfloat16).cuda() for _ in range(cp)]
+    ins_s = [torch.stack((torch.randn(tokens, cp, heads, generator=g) * 2,
+                          1 + torch.rand(tokens, cp, heads, generator=g) * 50), -1)
+             .reshape(tokens, cp, 2 * heads).contiguous().cuda() for _ in range(cp)]
+    ins_s[5][3, 7, 0] = float("-inf")      # one sender masked for one head
+    for channels in (0, 3):
+        combined, lse = hx.alltoall_combine_loopback(ins_o, ins_s, ws, hx.STATS_MAX_SUM, return_lse=True,
+                                                     channel_count=channels)
+        torch.cuda.synchronize()
+        assert ops.device_status() == 0
+        check(combined, lse, oracle_combine(ins_o, ins_s, heads, 1, ho.bf16_bits_to_f32), "bf16")
 
 
 def test_combine_while_senders_are_still_writing(hx, ops):
