@@ -408,8 +408,10 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
           }
           // statistics sit at the end of a message: few accesses touch the second tensor
           if (__ballot((o.a1 != kOutOfRange) | (o.b1 != kOutOfRange)) != 0ull) {
-            __builtin_amdgcn_raw_buffer_store_b64(wa, st.field1, o.a1, 0, kAuxNt);
-            __builtin_amdgcn_raw_buffer_store_b64(wb, st.field1, o.b1, 0, kAuxNt);
+            // (no streaming hint: a statistics row can be as small as 8 bytes, and the rows of the
+            // cp senders share 64-byte sectors that the L2 should merge before they go to memory)
+            __builtin_amdgcn_raw_buffer_store_b64(wa, st.field1, o.a1, 0, kAuxNone);
+            __builtin_amdgcn_raw_buffer_store_b64(wb, st.field1, o.b1, 0, kAuxNone);
           }
         }
         if (__ballot(anyPending) == 0ull) break;
