@@ -708,3 +708,35 @@ def test_per_rank_calls_on_separate_streams(hx, ops):
         torch.cuda.synchronize()
         check_against_oracle(ins_o, ins_s, [a for a, _ in snap], [b for _, b in snap])
     assert_clean(ops)
+
+
+def test_per_rank_calls_replay_from_a_captured_graph(hx, ops):
+    # the reference's signature, one call per logical rank, captured once and replayed on fresh payload
+    cp, entries = 4, 64
+    ws = get_workspace(hx, cp)
+    g = torch.Generator().manual_seed(29)
+    ins_o = [torch.randn(entries, cp, 512, generator=g).to(torch.bfloat16).cuda() for _ in range(cp)]
+    ins_s = [torch.randn(entries, cp, 8, generator=g).cuda() for _ in range(cp)]
+
+    def run():
+        return [hx.alltoall(ins_o[r], ins_s[r], ws, cp_rank=r, cp_size=cp) for r in range(cp)]
+
+    for _ in range(2):
+        run()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = run()
+    torch.cuda.synchronize()
+    for _ in range(4):
+        for a, b in outs:
+            a.zero_()
+            b.zero_()
+        for t in ins_o:
+            t.add_(1.0)
+        eager = run()                     # eager work between the replays, on the same workspace
+        graph.replay()
+        torch.cuda.synchronize()
+        check_against_oracle(ins_o, ins_s, [a for a, _ in outs], [b for _, b in outs], with_numpy=False)
+        check_against_oracle(ins_o, ins_s, [a for a, _ in eager], [b for _, b in eager], with_numpy=False)
+    assert_clean(ops)
