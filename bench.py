@@ -33,8 +33,8 @@ PEAK_HBM_GBPS = 8000.0
 # the same counters of a plain copy kernel); keyed by (workload, channel count used). Filled in from
 # the summaries under profiles/ when they exist for the configuration that is being run.
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/helix_exchange_kernel_c3_hbm_traffic.md: 76 191 420 fetched + 74 352 270 written
-    ("c3", 128): 150_543_690,
+    # profiles/helix_exchange_kernel_c3_hbm_traffic.md: 76 179 748 fetched + 74 022 183 written
+    ("c3", 128): 150_201_931,
 }
 
 
