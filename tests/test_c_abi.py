@@ -205,3 +205,15 @@ def test_header_is_c_and_a_c_host_can_call_the_library(ops, tmp_path):
     assert build.returncode == 0, build.stdout + build.stderr
     run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
     assert run.returncode == 0 and "c_abi_smoke ok" in run.stdout, run.stdout + run.stderr
+
+
+def test_import_fails_loudly_without_the_library(tmp_path):
+    # no CPU fallback: a missing libhelix_a2a.so is an ImportError that says how to build it
+    import subprocess
+    import sys
+
+    code = "import sys; sys.path.insert(0, %r); import helix_a2a" % str(ROOT / "helix-a2a_amd")
+    env = dict(**__import__("os").environ, HELIX_A2A_LIBRARY=str(tmp_path / "libhelix_a2a.so"))
+    run = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=300)
+    assert run.returncode != 0
+    assert "ImportError" in run.stderr and "build.py" in run.stderr and "no CPU fallback" in run.stderr
