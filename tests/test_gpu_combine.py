@@ -221,6 +221,23 @@ def test_combine_every_units_in_flight_variant(hx, ops, cp, tokens):
     check(combined, lse, oracle_combine(ins_o, ins_s, heads, 1, ho.bf16_bits_to_f32), "bf16")
 
 
+def test_combine_beyond_fifo_capacity_runs_in_rounds(hx, ops):
+    # one channel, 66-piece messages: 232 per FIFO entry, 928 per round of four entries; 2000 tokens take three rounds
+    cp, tokens, heads, d = 2, 2000, 2, 128
+    ws = workspace(hx, cp)
+    g = torch.Generator().manual_seed(41)
+    ins_o = [torch.randn(tokens, cp, heads * d, generator=g).to(torch.bfloat16).cuda() for _ in range(cp)]
+    ins_s = [torch.stack((torch.randn(tokens, cp, heads, generator=g) * 2,
+                          1 + torch.rand(tokens, cp, heads, generator=g) * 50), -1)
+             .reshape(tokens, cp, 2 * heads).contiguous().cuda() for _ in range(cp)]
+    want = oracle_combine(ins_o, ins_s, heads, 1, ho.bf16_bits_to_f32)
+    for _ in range(2):          # twice: the step counters continue from where the rounds left them
+        combined, lse = hx.alltoall_combine_loopback(ins_o, ins_s, ws, hx.STATS_MAX_SUM, return_lse=True, channel_count=1)
+        torch.cuda.synchronize()
+        assert ops.device_status() == 0
+        check(combined, lse, want, "bf16")
+
+
 def test_combine_thirty_two_ranks(hx, ops):
     # the largest rank count: 32 senders per (message, head), two slots per sideways pass
     cp, tokens, heads, d = 32, 20, 2, 64
