@@ -156,6 +156,29 @@ def test_loopback_workloads(hx, ops, name):
     check_against_oracle(ins_o, ins_s, outs_o, outs_s, with_numpy=name in ("c1", "c2", "c5b", "c3"))
 
 
+@pytest.mark.parametrize("name", ["c3", "c4", "c5a"])
+def test_exchange_twice_is_the_identity(hx, ops, name):
+    # out[r][e, s] = in[s][e, r], so exchanging the result again returns every rank its own input; and the
+    # exchange only moves bytes: sums of the 64-bit words (plain and shifted) over all ranks do not change
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS[name]
+    ws = get_workspace(hx, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    once_o, once_s = hx.alltoall_loopback(ins_o, ins_s, ws)
+    back_o, back_s = hx.alltoall_loopback(once_o, once_s, ws)
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    for r in range(w.cp):
+        assert bits_equal(back_o[r], ins_o[r]) and bits_equal(back_s[r], ins_s[r])
+
+    def digest(ts):
+        words = torch.cat([t.contiguous().view(torch.int64).reshape(-1) for t in ts])
+        return tuple(int((words >> shift).sum()) for shift in (0, 8, 16, 32))
+
+    assert digest(ins_o) == digest(once_o) and digest(ins_s) == digest(once_s)
+
+
 @pytest.mark.parametrize("name", ["c1", "c5b", "c2"])
 def test_loopback_against_reference_model(hx, ops, ref_model, name):
     # the C restatement of the reference kernel, run on the same bits
