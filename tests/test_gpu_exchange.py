@@ -763,3 +763,28 @@ def test_per_rank_calls_replay_from_a_captured_graph(hx, ops):
         check_against_oracle(ins_o, ins_s, [a for a, _ in outs], [b for _, b in outs], with_numpy=False)
         check_against_oracle(ins_o, ins_s, [a for a, _ in eager], [b for _, b in eager], with_numpy=False)
     assert_clean(ops)
+
+
+def test_reference_environment_switches(hx, ops, monkeypatch):
+    # HELIX_A2A_ENABLE_PDL (csrc/helix_alltoall.cu:541-548) is accepted and changes nothing: ordering between
+    # calls is stream order. HELIX_A2A_CHANNEL_COUNT (csrc/torch_binding.cpp:25-32) is honoured, re-read per call.
+    cp = 4
+    ws = get_workspace(hx, cp)
+    g = torch.Generator().manual_seed(31)
+    ins_o = [torch.randn(40, cp, 256, generator=g).to(torch.bfloat16).cuda() for _ in range(cp)]
+    ins_s = [torch.randn(40, cp, 4, generator=g).cuda() for _ in range(cp)]
+    for pdl in ("0", "1"):
+        monkeypatch.setenv("HELIX_A2A_ENABLE_PDL", pdl)
+        for channels in ("", "3", "40", "1"):
+            if channels:
+                monkeypatch.setenv("HELIX_A2A_CHANNEL_COUNT", channels)
+            else:
+                monkeypatch.delenv("HELIX_A2A_CHANNEL_COUNT", raising=False)
+            outs = [hx.alltoall(ins_o[r], ins_s[r], ws, cp_rank=r, cp_size=cp) for r in range(cp)]
+            torch.cuda.synchronize()
+            check_against_oracle(ins_o, ins_s, [a for a, _ in outs], [b for _, b in outs], with_numpy=False)
+    monkeypatch.setenv("HELIX_A2A_CHANNEL_COUNT", "100000")      # more than the layout provides
+    with pytest.raises(RuntimeError, match="max_channel_count"):
+        hx.alltoall(ins_o[0], ins_s[0], ws, cp_rank=0, cp_size=cp)
+    ops.reset_logical_ranks()
+    assert_clean(ops)
