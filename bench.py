@@ -247,6 +247,7 @@ def main() -> int:
         torch.cuda.synchronize()
 
     achieved = bytes_per_call / (avg_kernel_ms * 1e-3) / 1e9
+    traffic = None if (args.combine or args.layout == "head") else MEASURED_TRAFFIC_BYTES.get((w.name, channels))
     result = {
         "metric": METRIC,
         "value": bytes_per_call / (ms_per_step * 1e-3) / 1e9,
@@ -290,7 +291,9 @@ def main() -> int:
             "peak": PEAK_HBM_GBPS,
             "unit": "GB/s",
             "frac": achieved / PEAK_HBM_GBPS,
-            "traffic": None if (args.combine or args.layout == "head") else MEASURED_TRAFFIC_BYTES.get((w.name, channels)),
+            "traffic": traffic,
+            # the same fraction with the counted HBM traffic (FETCH_SIZE + WRITE_SIZE) in place of the algorithmic bytes
+            "frac_of_peak_from_counters": None if traffic is None else traffic / (avg_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
         },
     }
     if not args.no_cpu_baseline and not args.combine and args.layout == "token":
