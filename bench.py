@@ -29,12 +29,13 @@ for _p in (ROOT / "helix-a2a_amd", ROOT):
 METRIC = "µs/call + effective HBM GB/s (% of peak) for Helix a2a, cp=4/8, 1 GPU"
 PEAK_HBM_GBPS = 8000.0
 
-# HBM traffic per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE runs, scaled by
-# the same counters of a plain copy kernel); keyed by (workload, channel count used). Filled in from
-# the summaries under profiles/ when they exist for the configuration that is being run.
+# Bytes that crossed between the L2s and the fabric per launch (FETCH_SIZE + WRITE_SIZE of two
+# rocprofv3 --pmc runs, each scaled by the same counter of a plain copy kernel), one row per profiled
+# configuration: (kernel, workload, channels) -> bytes. The summaries under profiles/ named
+# <kernel>_<workload>_hbm_traffic.md hold the runs these come from. These counters sit between L2
+# and fabric: they do not tell whether the memory-side cache or DRAM served a request.
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/helix_exchange_kernel_c3_hbm_traffic.md: 76 179 748 fetched + 74 022 183 written
-    ("c3", 128): 150_201_931,
+    ("helix_exchange_kernel", "c3", 128): 150_201_931,
 }
 
 
@@ -110,6 +111,47 @@ def cpu_baseline(w, algorithmic_bytes: int, budget_s: float = 12.0):
     }
 
 
+def host_timing(w, ws, ins_o, ins_s, calls: int = 200):
+    """Host time of the drop-in calls: wall time of the Python call(s) that enqueue one exchange of all ranks,
+    with the GPU idle before and drained after each sample (so nothing waits for the device inside the call)."""
+    import torch
+
+    import helix_a2a
+
+    hp, d = w.heads_per_rank, w.head_dim
+    attn_out = [t.reshape(w.tokens, w.cp * hp, d) for t in ins_o]
+    attn_lse = [torch.randn(w.tokens, w.cp * hp, device="cuda") for _ in range(w.cp)]
+    lse_ok = hp % 2 == 0
+
+    def per_rank():
+        for r in range(w.cp):
+            helix_a2a.alltoall(ins_o[r], ins_s[r], ws, r, w.cp)
+
+    def loopback():
+        helix_a2a.alltoall_loopback(ins_o, ins_s, ws)
+
+    def reduce():
+        helix_a2a.dcp_a2a_lse_reduce(attn_out, attn_lse, ws)
+
+    out = {}
+    for name, fn in (("alltoall_x_cp", per_rank), ("alltoall_loopback", loopback)) + ((("dcp_a2a_lse_reduce", reduce),) if lse_ok else ()):
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+        samples = []
+        for _ in range(calls):
+            t0 = time.perf_counter()
+            fn()
+            samples.append(time.perf_counter() - t0)
+            torch.cuda.synchronize()
+        samples.sort()
+        out[name] = {"p50": percentile(samples, 0.5) * 1e6, "p5": percentile(samples, 0.05) * 1e6,
+                     "p95": percentile(samples, 0.95) * 1e6}
+    out["note"] = (f"alltoall_x_cp = {w.cp} calls of helix_a2a.alltoall (the reference's signature), one per logical rank; "
+                   "each figure is the wall time of the Python call(s) alone, GPU idle before and drained after")
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -123,6 +165,13 @@ def main() -> int:
                          "(token, head), stats are one float2 -- the layout the reference's serving integration passes")
     ap.add_argument("--graph", type=int, default=0, metavar="G",
                     help="replay the calls from a captured HIP graph of G calls (steps must be a multiple of G)")
+    ap.add_argument("--rotate", type=int, default=-1, metavar="N",
+                    help="sets of input and output tensors the cold leg cycles through (every step takes the next "
+                         "set, so the working set exceeds the 256 MB memory-side cache); -1 = as many as make "
+                         "1 GiB of tensors, 0 = no cold leg")
+    ap.add_argument("--units-per-wavefront", type=int, default=None, metavar="U",
+                    help="share runs longer than U KiB per wavefront between wavefronts (library default: 6; 0 = never)")
+    ap.add_argument("--no-host-timing", action="store_true", help="skip the host-time-per-call measurements")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
@@ -148,6 +197,8 @@ def main() -> int:
     ws = helix_a2a.allocate_workspace(w.cp, 0)
     for r in range(w.cp):
         helix_a2a.init_workspace(ws, r, w.cp)
+    if args.units_per_wavefront is not None:
+        _ops.set_units_per_wavefront(args.units_per_wavefront)
     ins_o, ins_s = make_inputs(w, "cuda")
     entries = w.tokens
     if args.layout == "head":
@@ -157,10 +208,12 @@ def main() -> int:
         pairs = [as_head_layout(w, o, s) for o, s in zip(ins_o, ins_s)]
         ins_o, ins_s = [p[0] for p in pairs], [p[1] for p in pairs]
         entries = w.tokens * w.heads_per_rank
-    if args.combine:
-        plan = _ops.CombinePlan(ins_o, ins_s, ws, _ops.STATS_MAX_SUM, False, args.channels)
-    else:
-        plan = _ops.LoopbackPlan(ins_o, ins_s, ws, args.channels)
+    def make_plan(o, s_):
+        if args.combine:
+            return _ops.CombinePlan(o, s_, ws, _ops.STATS_MAX_SUM, False, args.channels)
+        return _ops.LoopbackPlan(o, s_, ws, args.channels)
+
+    plan = make_plan(ins_o, ins_s)
     channels = args.channels or _ops.auto_channel_count(w.cp, entries)
     # algorithmic bytes: payload read + lines written + lines read + output written, with the lines this
     # channel count makes (the messages of a run are packed piece by piece, whole lines per run)
@@ -215,6 +268,32 @@ def main() -> int:
     status |= _ops.device_status()
     kernel_ms = sorted(s.elapsed_time(e) for s, e in zip(starts, ends))
 
+    # Cold leg: the same K steps, every step on the next of N sets of input and output tensors (same
+    # values, own memory), so that nothing a step touches is left in the memory-side cache from the
+    # step before; the FIFO entries rotate through their four positions as they always do.
+    cold = None
+    tensor_bytes = sum(t.numel() * t.element_size() for t in ins_o + ins_s) * 2
+    n_sets = args.rotate if args.rotate >= 0 else max(2, -(-(1 << 30) // tensor_bytes))
+    if n_sets >= 2 and graph is None:
+        plans = [plan] + [make_plan([t.clone() for t in ins_o], [t.clone() for t in ins_s]) for _ in range(n_sets - 1)]
+        for i in range(max(args.warmup, n_sets)):
+            plans[i % n_sets].run()
+        cold_start = torch.cuda.Event(enable_timing=True)
+        cold_end = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        cold_start.record()
+        for i in range(args.steps):
+            plans[i % n_sets].run()
+        cold_end.record()
+        torch.cuda.synchronize()
+        cold_wall = time.perf_counter() - t0
+        status |= _ops.device_status()
+        cold = {"sets": n_sets, "tensor_bytes_in_rotation": n_sets * tensor_bytes,
+                "kernel_us": cold_start.elapsed_time(cold_end) / args.steps * 1e3,
+                "us_per_call": cold_wall * 1e6 / args.steps}
+        del plans
+
     ok = status == 0
     if not args.no_check and args.combine:
         import numpy as np
@@ -247,7 +326,10 @@ def main() -> int:
         torch.cuda.synchronize()
 
     achieved = bytes_per_call / (avg_kernel_ms * 1e-3) / 1e9
-    traffic = None if (args.combine or args.layout == "head") else MEASURED_TRAFFIC_BYTES.get((w.name, channels))
+    kernel_name = "helix_combine_kernel" if args.combine else "helix_exchange_kernel"
+    traffic = None if args.layout == "head" else MEASURED_TRAFFIC_BYTES.get((kernel_name, w.name, channels))
+    # the exchange as a user sees it: payload in, payload out (a direct permuted copy would move just that)
+    useful_bytes = (w.payload_bytes + w.cp * w.tokens * w.field0_bytes) if args.combine else 2 * w.payload_bytes
     result = {
         "metric": METRIC,
         "value": bytes_per_call / (ms_per_step * 1e-3) / 1e9,
@@ -276,6 +358,9 @@ def main() -> int:
             "payload_bytes": w.payload_bytes, "wire_bytes": wire,
         },
         "kernel_us_in_timed_region": avg_kernel_ms * 1e3,
+        # payload read + result written over the time per call: what a direct permuted copy would have to move;
+        # `value` counts the FIFO write and read-back as well (the protocol's own traffic)
+        "payload_GBps": useful_bytes / (ms_per_step * 1e-3) / 1e9,
         "single_call_us": {
             "mean": statistics.fmean(kernel_ms) * 1e3,
             "p50": percentile(kernel_ms, 0.5) * 1e3,
@@ -286,7 +371,7 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "helix_combine_kernel" if args.combine else "helix_exchange_kernel",
+            "kernel": kernel_name,
             "achieved": achieved,
             "peak": PEAK_HBM_GBPS,
             "unit": "GB/s",
@@ -294,8 +379,15 @@ def main() -> int:
             "traffic": traffic,
             # the same fraction with the counted HBM traffic (FETCH_SIZE + WRITE_SIZE) in place of the algorithmic bytes
             "frac_of_peak_from_counters": None if traffic is None else traffic / (avg_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+            # `frac` re-uses one set of tensors every step (working set c3: 220 MB, inside the 256 MB memory-side
+            # cache); `frac_cold` cycles through `cold.sets` sets, so every step's tensors come from DRAM
+            "frac_cold": None if cold is None else bytes_per_call / (cold["kernel_us"] * 1e-6) / 1e9 / PEAK_HBM_GBPS,
+            "achieved_cold": None if cold is None else bytes_per_call / (cold["kernel_us"] * 1e-6) / 1e9,
         },
+        "cold": cold,
     }
+    if not args.no_host_timing and not args.combine and args.layout == "token" and graph is None:
+        result["host_us_per_call"] = host_timing(w, ws, ins_o, ins_s)
     if not args.no_cpu_baseline and not args.combine and args.layout == "token":
         result["cpu_baseline"] = cpu_baseline(w, bytes_per_call)
     print(json.dumps(result))

@@ -38,8 +38,13 @@ def find_hipcc() -> str:
     raise RuntimeError("hipcc not found (set HIPCC or install ROCm)")
 
 
-def build_library(verbose: bool = True) -> Path:
-    cmd = [find_hipcc(), *HIPCC_FLAGS, *map(str, SOURCES), "-o", str(OUTPUT)]
+TIMELINE_OUTPUT = HERE / "helix_a2a" / "libhelix_a2a_timeline.so"
+
+
+def build_library(verbose: bool = True, timeline: bool = False) -> Path:
+    """The library; with ``timeline`` the measuring variant whose kernels stamp their phases (a file of its own)."""
+    output = TIMELINE_OUTPUT if timeline else OUTPUT
+    cmd = [find_hipcc(), *HIPCC_FLAGS, *(["-DHELIX_A2A_TIMELINE"] if timeline else []), *map(str, SOURCES), "-o", str(output)]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -49,10 +54,10 @@ def build_library(verbose: bool = True) -> Path:
         print(log, flush=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed with exit code {proc.returncode}\n{log}")
-    return OUTPUT
+    return output
 
 
 if __name__ == "__main__":
-    build_library()
-    print(f"built {OUTPUT}")
+    out = build_library(timeline="--timeline" in sys.argv[1:])
+    print(f"built {out}")
     sys.exit(0)

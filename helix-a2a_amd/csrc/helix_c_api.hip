@@ -40,6 +40,24 @@ int fail(int code, const char* fmt, ...) {
 
 std::atomic<uint64_t> g_spinLimitUs{2000000};
 std::atomic<int> g_singleRound{0};
+// Units per lane a wavefront takes of a run before the run is shared with another wavefront:
+// -1 = kMaxUnitsInFlight, and only while the launch leaves wavefront slots of the device free;
+// 0 = never share; 1..6 = always share beyond that many.
+std::atomic<int> g_unitsPerWavefront{-1};
+
+// Wavefronts per stream a launch may use at most. The automatic rule looks at the whole exchange (both
+// directions of all cp ranks), not at the launch, so that the send and receive halves of one exchange
+// cut their runs the same way even when they are issued as separate launches of different extent.
+int max_parts_for(const KernelArgs& a, int cuCount) {
+  const int mode = g_unitsPerWavefront.load();
+  if (mode == 0) return 1;
+  if (mode > 0) return kMaxStreamParts;
+  return auto_max_parts(a.cpSize, a.runChannels, cuCount);
+}
+int units_per_part() {
+  const int mode = g_unitsPerWavefront.load();
+  return mode > 0 ? mode : kMaxUnitsInFlight;
+}
 
 constexpr int kMaxDevices = 64;
 struct DeviceState {
@@ -116,6 +134,13 @@ int env_channel_count() {
   return v > 0 ? v : 0;
 }
 
+// A workspace the library provides itself, in place of the descriptor's.
+struct BuiltinWorkspace {
+  uint8_t* base;
+  uint64_t rowStrideBytes;
+  int maxChannels;
+};
+
 struct Plan {
   KernelArgs args;
   int entryCount;
@@ -147,7 +172,8 @@ int check_field(const helix_a2a_field_t& f, const char* name, int eltSize, int e
 // kernel argument block. Checks that need no device come first, so that a
 // malformed descriptor is reported even where no GPU is present. `exchangeOutputs` selects whether recv_fields are
 // checked (exchange) or ignored (combine).
-int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs, Plan* plan) {
+int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs, Plan* plan,
+               const BuiltinWorkspace* builtin = nullptr) {
   if (ranks == nullptr || count < 1) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "no rank descriptors given");
   const helix_a2a_params_t& p0 = ranks[0];
   int rc = check_cp_size(p0.cp_size);
@@ -155,9 +181,14 @@ int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs,
   const int cp = p0.cp_size;
   if (count > cp) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%d rank descriptors for cp_size %d", count, cp);
   if (p0.entry_count < 0) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "entry_count must be >= 0");
-  if (p0.workspace == nullptr) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace pointer is null");
-  if ((reinterpret_cast<uintptr_t>(p0.workspace) % kUnitBytes) != 0 || (p0.workspace_stride_u64 % 2) != 0)
-    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace rows must be 16-byte aligned");
+  if (builtin != nullptr) {
+    if (p0.workspace != nullptr)
+      return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "the workspace pointer must be null: this call uses the built-in workspace");
+  } else {
+    if (p0.workspace == nullptr) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace pointer is null");
+    if ((reinterpret_cast<uintptr_t>(p0.workspace) % kUnitBytes) != 0 || (p0.workspace_stride_u64 % 2) != 0)
+      return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace rows must be 16-byte aligned");
+  }
 
   KernelArgs a;
   std::memset(&a, 0, sizeof(a));
@@ -214,25 +245,33 @@ int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs,
   int cuCount = 0;
   rc = resolve_cu_count(0, &cuCount);
   if (rc) return rc;
-  const int maxCh = max_channel_count(cp, cuCount);
-  if (p0.max_channel_count != maxCh)
-    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "max_channel_count %d does not match the device's %d (cp_size %d, %d CUs)",
-                p0.max_channel_count, maxCh, cp, cuCount);
-  if (p0.workspace_stride_u64 * 8ull < workspace_bytes(cp, maxCh))
-    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace row of %llu bytes is smaller than the %llu bytes cp_size %d needs",
-                static_cast<unsigned long long>(p0.workspace_stride_u64 * 8ull),
-                static_cast<unsigned long long>(workspace_bytes(cp, maxCh)), cp);
+  const int maxCh = builtin ? builtin->maxChannels : max_channel_count(cp, cuCount);
+  if (builtin == nullptr) {
+    if (p0.max_channel_count != maxCh)
+      return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "max_channel_count %d does not match the device's %d (cp_size %d, %d CUs)",
+                  p0.max_channel_count, maxCh, cp, cuCount);
+    if (p0.workspace_stride_u64 * 8ull < workspace_bytes(cp, maxCh))
+      return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "workspace row of %llu bytes is smaller than the %llu bytes cp_size %d needs",
+                  static_cast<unsigned long long>(p0.workspace_stride_u64 * 8ull),
+                  static_cast<unsigned long long>(workspace_bytes(cp, maxCh)), cp);
+  }
 
   int channels = p0.channel_count > 0 ? p0.channel_count : env_channel_count();
-  if (channels > maxCh)
-    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "channel_count %d exceeds max_channel_count %d", channels, maxCh);
-  if (channels <= 0) channels = auto_channels(cp, p0.entry_count, cuCount);
+  if (channels > maxCh) {
+    if (p0.channel_count > 0 || builtin == nullptr)
+      return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "channel_count %d exceeds max_channel_count %d", channels, maxCh);
+    channels = maxCh;  // the environment's count is a wish, and the built-in workspace is smaller than a caller's
+  }
+  if (channels <= 0) {
+    channels = auto_channels(cp, p0.entry_count, cuCount);
+    if (channels > maxCh) channels = maxCh;
+  }
 
   DeviceState* st = nullptr;
   if ((rc = device_state(&st))) return rc;
 
-  a.workspace = reinterpret_cast<uint8_t*>(p0.workspace);
-  a.rowStrideBytes = p0.workspace_stride_u64 * 8ull;
+  a.workspace = builtin ? builtin->base : reinterpret_cast<uint8_t*>(p0.workspace);
+  a.rowStrideBytes = builtin ? builtin->rowStrideBytes : p0.workspace_stride_u64 * 8ull;
   a.cpSize = cp;
   a.maxChannels = maxCh;
   a.runChannels = channels;
@@ -282,14 +321,14 @@ int launch_rounds(Plan& plan, bool send, bool recv, bool allowRounds, hipStream_
     long waves = 2L * waves_per_direction(a);
     if (waves > static_cast<long>(plan.cuCount) * 8)
       return fail(HELIX_A2A_ERR_CAPACITY, "single-round launch of %ld wavefronts is not guaranteed co-resident", waves);
-    HELIX_HIP_TRY(launch_exchange(a, stream));
+    HELIX_HIP_TRY(launch_exchange(a, kMaxUnitsInFlight, 1, stream));  // senders wait on the one tail counter: one wavefront per stream
     return HELIX_A2A_OK;
   }
   for (int begin = 0; begin < plan.entryCount; begin += plan.roundEntries) {
     a.entryBegin = begin;
     long end = static_cast<long>(begin) + plan.roundEntries;
     a.entryEnd = end > plan.entryCount ? plan.entryCount : static_cast<int>(end);
-    HELIX_HIP_TRY(launch_exchange(a, stream));
+    HELIX_HIP_TRY(launch_exchange(a, units_per_part(), max_parts_for(a, plan.cuCount), stream));
   }
   return HELIX_A2A_OK;
 }
@@ -450,6 +489,14 @@ int helix_a2a_device_status(uint32_t* status, void* stream) {
 void helix_a2a_set_spin_limit_us(uint64_t microseconds) { g_spinLimitUs.store(microseconds); }
 
 void helix_a2a_set_single_round(int enabled) { g_singleRound.store(enabled ? 1 : 0); }
+
+
+int helix_a2a_set_units_per_wavefront(int units) {
+  if (units < -1 || units > kMaxUnitsInFlight)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "units per wavefront must be in [-1, %d], got %d", kMaxUnitsInFlight, units);
+  g_unitsPerWavefront.store(units);
+  return HELIX_A2A_OK;
+}
 
 const char* helix_a2a_last_error(void) { return g_lastError; }
 

@@ -2,13 +2,28 @@
 //
 // One wavefront owns one stream = (sender rank, receiver rank, channel) in one
 // direction, the role a warp has in the reference kernel
-// (csrc/helix_alltoall.cu:315-474). A sender wavefront reads its messages from
-// the send tensors, turns them into LL128 lines in registers and stores the
-// lines into the receiver's FIFO; a receiver wavefront polls the FIFO lines
-// until their flags carry the expected step, then stores the payload into the
+// (csrc/helix_alltoall.cu:315-474); a long run in a launch that leaves the device
+// under-filled is shared by several wavefronts, each with a slice of its own.
+// A sender wavefront reads its messages from the send tensors, turns them into
+// LL128 lines in registers, stores the lines into the receiver's FIFO and, once
+// those stores are acknowledged, moves its step counter: that is the token its
+// receiver waits for. A receiver wavefront then reads the lines in one pass,
+// checks that their flags carry the step, and stores the payload into the
 // receive tensors. There is no staging copy and no barrier: data moves
 // global -> registers -> FIFO -> registers -> global, 16 bytes per lane on
 // the FIFO side.
+//
+// Why the token and not the flags alone: a 64-lane 16-byte load of eight lines
+// is served in 64-byte halves, and the flag word of a line sits in its second
+// half. A receiver that reads a line while it is being written can see a
+// valid flag next to a stale first half. The counter moves only after the
+// sender has waited for every store of the step (s_waitcnt vmcnt(0) on
+// write-through stores), so a line is never read before all of it is in
+// memory, whatever the granularity of the memory system. Measured on MI355X
+// the token costs nothing against polling the flags (within 0.5 % on every
+// workload): sender wavefronts are dispatched first, so receivers rarely start
+// before their run is complete. The flags stay in the line format and are
+// still compared: a mismatch after the token means a corrupt workspace.
 //
 // The messages a stream puts into one FIFO entry form a "run": they follow
 // each other without gaps from line 0 of the entry, so a wavefront walks a
@@ -21,9 +36,9 @@
 // and drops stores that would fall outside, and an offset of kOutOfRange is
 // how a lane opts out of an access without a branch.
 //
-// FIFO lines are written and polled with the sc1 cache policy (device-scope
-// coherence: every XCD has its own L2, and the sender and the receiver of a
-// stream may run on different XCDs).
+// FIFO lines and counters are written and read with the sc1 cache policy
+// (device-scope coherence: every XCD has its own L2, and the sender and the
+// receiver of a stream may run on different XCDs).
 #include "helix_kernels.hpp"
 
 #include <hip/hip_fp16.h>
@@ -72,6 +87,26 @@ __device__ __forceinline__ int64_t ld_counter(const int64_t* p) {
 __device__ __forceinline__ void st_counter(int64_t* p, int64_t v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+
+// Phase stamps. A build with -DHELIX_A2A_TIMELINE (build.py --timeline, a separate library file) makes
+// every wavefront record the 100 MHz clock at four points of its program: 0 start, 1 its input is in
+// registers (sender: payload and counters; receiver: token seen and lines loaded), 2 its stores are
+// issued, 3 done (sender: stores acknowledged). The stamped build waits for outstanding memory
+// operations at points 1 and 3, which the product build does not; it is a measuring tool only.
+#ifdef HELIX_A2A_TIMELINE
+constexpr int kTimelineWaves = 1 << 16;
+__device__ uint64_t g_timeline[kTimelineWaves * 4];
+#define HELIX_MARK(wave, k, drain)                                                                 \
+  do {                                                                                             \
+    if (drain) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                    \
+    if (lane == 0 && (wave) >= 0 && (wave) < kTimelineWaves)                                       \
+      g_timeline[(wave) * 4 + (k)] = __builtin_amdgcn_s_memrealtime();                             \
+  } while (0)
+#else
+#define HELIX_MARK(wave, k, drain) \
+  do {                            \
+  } while (0)
+#endif
 
 // Bounded wait bookkeeping. The clock is read every 64th spin only.
 struct SpinGuard {
@@ -166,14 +201,17 @@ __device__ __forceinline__ UnitOffsets unit_offsets(const Stream& st, uint32_t f
 // ---------------------------------------------------------------------------
 // sender
 // ---------------------------------------------------------------------------
+// Part `part` of the a.parts wavefronts that send stream (s -> r, ch): it walks its slice of every run.
 template <int kAux, int kUnitsInFlight>
-__device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, int ch, int lane) {
+__device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, int ch, int part, int lane, int wave) {
+  HELIX_MARK(wave, 0, false);
   Stream st;
   setup_stream(st, a, r, ch);
   if (st.msgs == 0) return;
   uint8_t* senderRow = a.workspace + static_cast<uint64_t>(s) * a.rowStrideBytes;
   uint8_t* receiverRow = a.workspace + static_cast<uint64_t>(r) * a.rowStrideBytes;
   int64_t* info = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(a.cpSize, a.maxChannels, r, ch));
+  int64_t* token = info + sender_counter_slot(part);
   st.fifo = make_rsrc(receiverRow + fifo_offset(s, ch, a.maxChannels), kFifoBytes);
   st.field0 = make_rsrc(a.rank[s].send0, a.sendBytes0);
   st.field1 = make_rsrc(a.rank[s].send1, a.sendBytes1);
@@ -181,19 +219,41 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
   st.stride1 = a.sendStride1;
 
   // the counters are only needed once the first payload loads are in flight
-  int64_t step = info[0];
+  int64_t step = *token;
   int64_t tail = info[1];
 
   for (int firstMsg = 0; firstMsg < st.msgs; firstMsg += st.msgsPerEntry) {
     const int runMsgs = min(st.msgsPerEntry, st.msgs - firstMsg);
     const uint32_t runUnits = stream_run_units(st, runMsgs);
-    for (uint32_t U0 = 0; U0 < runUnits; U0 += kUnitsInFlight * kWaveLanes) {
+    const Slice slice = slice_of_run(runUnits, part, a.parts);
+    bool opened = false;
+    // open the FIFO entry of this run (csrc/helix_alltoall.cu:377-390); false when the wait for room gave up
+    auto open_entry = [&]() -> bool {
+      opened = true;
+      if (firstMsg > 0) {
+        step += 1;
+        wait_stores_acknowledged();
+        if (lane == 0) st_counter(token, step);
+      }
+      SpinGuard guard(a.spinLimitTicks);
+      while (tail + kFifoDepth <= step) {  // the entry is free once the receiver released step - 4
+        tail = ld_counter(&info[1]);
+        if (tail + kFifoDepth > step) break;
+        if (guard.expired()) {
+          raise_status(a.status, kStatusSendTimeout, lane);
+          return false;
+        }
+        __builtin_amdgcn_s_sleep(4);
+      }
+      return true;
+    };
+    for (uint32_t U0 = slice.begin; U0 < slice.end; U0 += kUnitsInFlight * kWaveLanes) {
       u32x2 wa[kUnitsInFlight], wb[kUnitsInFlight];
       unsigned long long needField1[kUnitsInFlight];  // wave-uniform: lanes of access i that hold statistics pieces
 #pragma unroll
       for (int i = 0; i < kUnitsInFlight; ++i) {
         uint32_t U = U0 + i * kWaveLanes + lane;
-        UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < runUnits);
+        UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < slice.end);
         wa[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field0, o.a0, 0, kAuxNone);
         wb[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field0, o.b0, 0, kAuxNone);
         needField1[i] = __ballot((o.a1 != kOutOfRange) | (o.b1 != kOutOfRange));
@@ -207,7 +267,7 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
         sb[i] = u32x2{0u, 0u};
         if (needField1[i] != 0ull) {
           uint32_t U = U0 + i * kWaveLanes + lane;
-          UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < runUnits);
+          UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < slice.end);
           sa[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.a1, 0, kAuxNone);
           sb[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.b1, 0, kAuxNone);
         }
@@ -217,24 +277,8 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
         wa[i] |= sa[i];
         wb[i] |= sb[i];
       }
-      if (U0 == 0) {
-        // open the FIFO entry of this run (csrc/helix_alltoall.cu:377-390)
-        if (firstMsg > 0) {
-          step += 1;
-          wait_stores_acknowledged();
-          if (lane == 0) st_counter(&info[0], step);
-        }
-        SpinGuard guard(a.spinLimitTicks);
-        while (tail + kFifoDepth <= step) {  // the entry is free once the receiver released step - 4
-          tail = ld_counter(&info[1]);
-          if (tail + kFifoDepth > step) break;
-          if (guard.expired()) {
-            raise_status(a.status, kStatusSendTimeout, lane);
-            return;
-          }
-          __builtin_amdgcn_s_sleep(4);
-        }
-      }
+      if (!opened && !open_entry()) return;
+      if (U0 == slice.begin && firstMsg == 0) HELIX_MARK(wave, 1, true);
       const uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
       const uint32_t stepLo = static_cast<uint32_t>(step);
       const uint32_t stepHi = static_cast<uint32_t>(static_cast<uint64_t>(step) >> 32);
@@ -243,20 +287,30 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
         uint32_t U = U0 + i * kWaveLanes + lane;
         bool flag = (U & 7u) == 7u;
         u32x4 v = {wa[i].x, wa[i].y, flag ? stepLo : wb[i].x, flag ? stepHi : wb[i].y};
-        uint32_t off = U < runUnits ? entryOffset + U * kUnitBytes : kOutOfRange;
+        uint32_t off = U < slice.end ? entryOffset + U * kUnitBytes : kOutOfRange;
         __builtin_amdgcn_raw_buffer_store_b128(v, st.fifo, off, 0, kAux);
       }
     }
+    if (!opened && !open_entry()) return;  // nothing of this run falls to this part: the step still counts
   }
+  // Close the last entry (csrc/helix_alltoall.cu:409-412): once this part's stores are acknowledged its
+  // counter moves beyond the step, which tells the receiving part that every line of the slice is in memory.
+  HELIX_MARK(wave, 2, false);
   wait_stores_acknowledged();
-  if (lane == 0) st_counter(&info[0], step + 1);  // close the last entry (csrc/helix_alltoall.cu:409-412)
+  HELIX_MARK(wave, 3, false);
+  if (lane == 0) st_counter(token, step + 1);
 }
 
 // ---------------------------------------------------------------------------
 // receiver
 // ---------------------------------------------------------------------------
+// Part `part` of the wavefronts that receive stream (s -> r, ch). It waits for the token of the sending
+// part (that part's counter beyond the step: all its lines of the step are in memory), reads its slice
+// in passes of kUnitsInFlight units per lane and stores the payload. Line flags are still compared: one
+// that disagrees after the token means the workspace is corrupt.
 template <int kAux, int kUnitsInFlight, bool kAlignedStores>
-__device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, int ch, int lane) {
+__device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, int ch, int part, int lane, int wave) {
+  HELIX_MARK(wave, 0, false);
   Stream st;
   setup_stream(st, a, s, ch);
   if (st.msgs == 0) return;
@@ -264,207 +318,176 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
   uint8_t* receiverRow = a.workspace + static_cast<uint64_t>(r) * a.rowStrideBytes;
   int64_t* senderInfo = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(a.cpSize, a.maxChannels, r, ch));
   int64_t* info = reinterpret_cast<int64_t*>(receiverRow + receiver_info_offset(a.cpSize, a.maxChannels, s, ch));
+  int64_t* token = senderInfo + sender_counter_slot(part);
+  int64_t* mine = info + receiver_counter_slot(part);
   st.fifo = make_rsrc(receiverRow + fifo_offset(s, ch, a.maxChannels), kFifoBytes);
   st.field0 = make_rsrc(a.rank[r].recv0, a.recvBytes0);
   st.field1 = make_rsrc(a.rank[r].recv1, a.recvBytes1);
   st.stride0 = a.recvStride0;
   st.stride1 = a.recvStride1;
 
-  int64_t step = info[1];
-  // The sender's head is the acquire token of a whole run: once it is beyond
-  // `step`, every line of that step is in memory (the sender waits for its
-  // stores before it moves head) and the run can be read in one pass.
-  int64_t head = ld_counter(&senderInfo[0]);
-  const int flagLane = lane | 7;
+  int64_t step = *mine;
+  int64_t head = ld_counter(token);
 
   for (int firstMsg = 0; firstMsg < st.msgs; firstMsg += st.msgsPerEntry) {
     const int runMsgs = min(st.msgsPerEntry, st.msgs - firstMsg);
     const uint32_t runUnits = stream_run_units(st, runMsgs);
+    const Slice slice = slice_of_run(runUnits, part, a.parts);
     if (firstMsg > 0) {
-      // every line of the previous entry has been consumed: hand it back to
-      // the sender (csrc/helix_alltoall.cu:427-449)
+      // this part's lines of the previous entry have been consumed (csrc/helix_alltoall.cu:427-449);
+      // part 0's counter is the tail the sender's back-pressure reads
       step += 1;
       if (lane == 0) {
-        st_counter(&info[1], step);
-        st_counter(&senderInfo[1], step);
+        st_counter(mine, step);
+        if (part == 0) st_counter(&senderInfo[1], step);
       }
-      if (head <= step) head = ld_counter(&senderInfo[0]);
     }
-    bool runClosed = head > step;
-    const uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
-    const uint32_t stepLo = static_cast<uint32_t>(step);
-    const uint32_t stepHi = static_cast<uint32_t>(static_cast<uint64_t>(step) >> 32);
-    for (uint32_t U0 = 0; U0 < runUnits; U0 += kUnitsInFlight * kWaveLanes) {
-      bool pending[kUnitsInFlight];
-#pragma unroll
-      for (int i = 0; i < kUnitsInFlight; ++i) pending[i] = (U0 + i * kWaveLanes + lane) < runUnits;
+    if (head <= step) {
       SpinGuard guard(a.spinLimitTicks);
       for (;;) {
-        bool landed[kUnitsInFlight];
-        if (runClosed) {
-#pragma unroll
-          for (int i = 0; i < kUnitsInFlight; ++i) landed[i] = pending[i];
-        } else {
-          // The sender may still be writing. Acquire line by line: first the flag
-          // words (upper half of each line's last unit, loaded by the eight flag
-          // lanes only), then -- with offsets that depend on what those loads
-          // returned -- the units of the lines whose flag carries the step. A unit
-          // is never read before its line's flag was seen, whatever the
-          // granularity at which the memory system serves a 128-byte line.
-          u32x2 f[kUnitsInFlight];
-#pragma unroll
-          for (int i = 0; i < kUnitsInFlight; ++i) {  // all flag loads first: one round trip, not one per access
-            uint32_t U = U0 + i * kWaveLanes + lane;
-            bool isFlagLane = (U & 7u) == 7u;
-            uint32_t off = (pending[i] && isFlagLane) ? entryOffset + U * kUnitBytes + kPieceBytes : kOutOfRange;
-            f[i] = __builtin_amdgcn_raw_buffer_load_b64(st.fifo, off, 0, kAux);
-          }
-#pragma unroll
-          for (int i = 0; i < kUnitsInFlight; ++i) {
-            uint32_t U = U0 + i * kWaveLanes + lane;
-            bool isFlagLane = (U & 7u) == 7u;
-            bool ok = !pending[i] || !isFlagLane || (f[i].x == stepLo && f[i].y == stepHi);
-            unsigned long long okMask = __ballot(ok);
-            landed[i] = pending[i] && ((okMask >> flagLane) & 1ull) != 0ull;
-          }
-        }
-        u32x4 v[kUnitsInFlight];
-#pragma unroll
-        for (int i = 0; i < kUnitsInFlight; ++i) {
-          uint32_t U = U0 + i * kWaveLanes + lane;
-          uint32_t off = landed[i] ? entryOffset + U * kUnitBytes : kOutOfRange;
-          v[i] = __builtin_amdgcn_raw_buffer_load_b128(st.fifo, off, 0, kAux);
-        }
-        // every unit that is consumed carries its line's flag in the very load that brought it
-        bool anyPending = false;
-        bool flagsAgree = true;
-#pragma unroll
-        for (int i = 0; i < kUnitsInFlight; ++i) {
-          uint32_t U = U0 + i * kWaveLanes + lane;
-          bool isFlagLane = (U & 7u) == 7u;
-          bool ok = !landed[i] || !isFlagLane || (v[i].z == stepLo && v[i].w == stepHi);
-          unsigned long long okMask = __ballot(ok);
-          bool lineOk = ((okMask >> flagLane) & 1ull) != 0ull;
-          flagsAgree &= !landed[i] || lineOk;
-          landed[i] = landed[i] && lineOk;
-          pending[i] = pending[i] && !landed[i];
-          anyPending |= pending[i];
-        }
-        const bool wholePass = runClosed && __ballot(!flagsAgree) == 0ull;  // every unit of the pass is here
-        if (!wholePass) runClosed = false;  // not what the token promised (or no token yet): go line by line
-        const bool store16s = kAlignedStores && wholePass;
-#pragma unroll
-        for (int i = 0; i < kUnitsInFlight; ++i) {
-          uint32_t U = U0 + i * kWaveLanes + lane;
-          RunUnit d;
-          UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, landed[i], &d);
-          u32x2 wa = {v[i].x, v[i].y};
-          u32x2 wb = {v[i].z, v[i].w};
-          if (store16s) {
-            // Messages follow each other piece by piece and a line carries 15 of
-            // them, so the two pieces of a unit sit astride a 16-byte boundary
-            // of the output row about half of the time, and the two 8-byte stores
-            // of an access then each write every other 8 bytes. With the whole
-            // pass in registers every lane stores the aligned 16 bytes ("chunk")
-            // that start at whichever of its words is an even partial_o piece:
-            //   first word even:   both own words, or -- in the flag unit -- the
-            //                      own word + the first word of the next unit;
-            //   second word even:  that word + the first word of the next unit;
-            // the next unit being the next lane (for lane 63, lane 0 of the next
-            // access). An odd first word belongs to the previous unit's chunk.
-            // Where the pass ends between the halves of a chunk, both are stored
-            // alone. (Costs a dozen vector instructions per unit and halves the
-            // store instructions: measured on MI355X it is 5-6 % faster on runs
-            // of several passes and 2 % slower on single-pass runs, hence a
-            // template parameter the host sets through KernelArgs::alignedStores.)
-            uint32_t nx = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v[i].x), kDppWaveShl1, 0xF, 0xF, false));
-            uint32_t ny = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v[i].y), kDppWaveShl1, 0xF, 0xF, false));
-            const bool haveNext = lane < kWaveLanes - 1 || i + 1 < kUnitsInFlight;
-            if (i + 1 < kUnitsInFlight) {
-              const uint32_t fx = lane_value(v[i + 1 < kUnitsInFlight ? i + 1 : i].x, 0);
-              const uint32_t fy = lane_value(v[i + 1 < kUnitsInFlight ? i + 1 : i].y, 0);
-              if (lane == kWaveLanes - 1) {
-                nx = fx;
-                ny = fy;
-              }
-            }
-            const bool startsAtA = o.a0 != kOutOfRange && (d.pieceA & 1u) == 0u;
-            const bool startsAtB = o.b0 != kOutOfRange && (d.pieceB & 1u) == 0u;
-            const bool takesNext = startsAtB || (startsAtA && d.flag);
-            const bool store16 = (startsAtA || startsAtB) && (!takesNext || haveNext);
-            u32x4 chunk = {startsAtB ? v[i].z : v[i].x, startsAtB ? v[i].w : v[i].y, takesNext ? nx : v[i].z,
-                           takesNext ? ny : v[i].w};
-            __builtin_amdgcn_raw_buffer_store_b128(chunk, st.field0, store16 ? (startsAtB ? o.b0 : o.a0) : kOutOfRange, 0,
-                                                   kAuxNt);
-            // the halves of a chunk the pass boundary separates: the last lane's flag unit, the first lane's first word
-            const bool alone = o.a0 != kOutOfRange &&
-                               ((i == kUnitsInFlight - 1 && lane == kWaveLanes - 1 && startsAtA && d.flag) ||
-                                (i == 0 && lane == 0 && (d.pieceA & 1u) != 0u));
-            if ((i == 0 || i == kUnitsInFlight - 1) && __ballot(alone) != 0ull)
-              __builtin_amdgcn_raw_buffer_store_b64(wa, st.field0, alone ? o.a0 : kOutOfRange, 0, kAuxNt);
-          } else {
-            __builtin_amdgcn_raw_buffer_store_b64(wa, st.field0, o.a0, 0, kAuxNt);
-            __builtin_amdgcn_raw_buffer_store_b64(wb, st.field0, o.b0, 0, kAuxNt);
-          }
-          // statistics sit at the end of a message: few accesses touch the second tensor
-          if (__ballot((o.a1 != kOutOfRange) | (o.b1 != kOutOfRange)) != 0ull) {
-            // (no streaming hint: a statistics row can be as small as 8 bytes, and the rows of the
-            // cp senders share 64-byte sectors that the L2 should merge before they go to memory)
-            __builtin_amdgcn_raw_buffer_store_b64(wa, st.field1, o.a1, 0, kAuxNone);
-            __builtin_amdgcn_raw_buffer_store_b64(wb, st.field1, o.b1, 0, kAuxNone);
-          }
-        }
-        if (__ballot(anyPending) == 0ull) break;
+        head = ld_counter(token);
+        if (head > step) break;
         if (guard.expired()) {
           raise_status(a.status, kStatusRecvTimeout, lane);
           return;
         }
         __builtin_amdgcn_s_sleep(1);
-        asm volatile("" ::: "memory");
+      }
+    }
+    asm volatile("" ::: "memory");  // no line is read before the token was seen
+    const uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
+    const uint32_t stepLo = static_cast<uint32_t>(step);
+    const uint32_t stepHi = static_cast<uint32_t>(static_cast<uint64_t>(step) >> 32);
+    for (uint32_t U0 = slice.begin; U0 < slice.end; U0 += kUnitsInFlight * kWaveLanes) {
+      const uint32_t passEnd = min(U0 + kUnitsInFlight * kWaveLanes, slice.end);
+      u32x4 v[kUnitsInFlight];
+#pragma unroll
+      for (int i = 0; i < kUnitsInFlight; ++i) {
+        uint32_t U = U0 + i * kWaveLanes + lane;
+        uint32_t off = U < passEnd ? entryOffset + U * kUnitBytes : kOutOfRange;
+        v[i] = __builtin_amdgcn_raw_buffer_load_b128(st.fifo, off, 0, kAux);
+      }
+      // every line carries its flag in the very load that brought its last unit
+      bool flagsAgree = true;
+#pragma unroll
+      for (int i = 0; i < kUnitsInFlight; ++i) {
+        uint32_t U = U0 + i * kWaveLanes + lane;
+        flagsAgree &= U >= passEnd || (U & 7u) != 7u || (v[i].z == stepLo && v[i].w == stepHi);
+      }
+      if (__ballot(!flagsAgree) != 0ull) {
+        raise_status(a.status, kStatusInternal, lane);
+        return;
+      }
+      if (U0 == slice.begin && firstMsg == 0) HELIX_MARK(wave, 1, false);
+#pragma unroll
+      for (int i = 0; i < kUnitsInFlight; ++i) {
+        uint32_t U = U0 + i * kWaveLanes + lane;
+        RunUnit d;
+        UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < passEnd, &d);
+        u32x2 wa = {v[i].x, v[i].y};
+        u32x2 wb = {v[i].z, v[i].w};
+        if (kAlignedStores) {
+          // Messages follow each other piece by piece and a line carries 15 of
+          // them, so the two pieces of a unit sit astride a 16-byte boundary
+          // of the output row about half of the time, and the two 8-byte stores
+          // of an access then each write every other 8 bytes. With the whole
+          // pass in registers every lane stores the aligned 16 bytes ("chunk")
+          // that start at whichever of its words is an even partial_o piece:
+          //   first word even:   both own words, or -- in the flag unit -- the
+          //                      own word + the first word of the next unit;
+          //   second word even:  that word + the first word of the next unit;
+          // the next unit being the next lane (for lane 63, lane 0 of the next
+          // access). An odd first word belongs to the previous unit's chunk.
+          // Where the pass ends between the halves of a chunk, both are stored
+          // alone. (Costs a dozen vector instructions per unit and halves the
+          // store instructions: measured on MI355X it is 5-6 % faster on long
+          // runs and 2 % slower on runs of one short pass, hence a template
+          // parameter the host sets through KernelArgs::alignedStores.)
+          uint32_t nx = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v[i].x), kDppWaveShl1, 0xF, 0xF, false));
+          uint32_t ny = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v[i].y), kDppWaveShl1, 0xF, 0xF, false));
+          const bool haveNext = U + 1u < passEnd;
+          if (i + 1 < kUnitsInFlight) {
+            const uint32_t fx = lane_value(v[i + 1 < kUnitsInFlight ? i + 1 : i].x, 0);
+            const uint32_t fy = lane_value(v[i + 1 < kUnitsInFlight ? i + 1 : i].y, 0);
+            if (lane == kWaveLanes - 1) {
+              nx = fx;
+              ny = fy;
+            }
+          }
+          const bool startsAtA = o.a0 != kOutOfRange && (d.pieceA & 1u) == 0u;
+          const bool startsAtB = o.b0 != kOutOfRange && (d.pieceB & 1u) == 0u;
+          const bool takesNext = startsAtB || (startsAtA && d.flag);
+          const bool store16 = (startsAtA || startsAtB) && (!takesNext || haveNext);
+          u32x4 chunk = {startsAtB ? v[i].z : v[i].x, startsAtB ? v[i].w : v[i].y, takesNext ? nx : v[i].z,
+                         takesNext ? ny : v[i].w};
+          __builtin_amdgcn_raw_buffer_store_b128(chunk, st.field0, store16 ? (startsAtB ? o.b0 : o.a0) : kOutOfRange, 0,
+                                                 kAuxNt);
+          // the halves of a chunk the pass boundary separates: the last unit's lone first word (a flag
+          // unit: passes end on line boundaries), the first unit's odd first word
+          const bool alone = o.a0 != kOutOfRange && ((U + 1u == passEnd && startsAtA && d.flag) ||
+                                                     (U == U0 && (d.pieceA & 1u) != 0u));
+          if (__ballot(alone) != 0ull)
+            __builtin_amdgcn_raw_buffer_store_b64(wa, st.field0, alone ? o.a0 : kOutOfRange, 0, kAuxNt);
+        } else {
+          __builtin_amdgcn_raw_buffer_store_b64(wa, st.field0, o.a0, 0, kAuxNt);
+          __builtin_amdgcn_raw_buffer_store_b64(wb, st.field0, o.b0, 0, kAuxNt);
+        }
+        // statistics sit at the end of a message: few accesses touch the second tensor
+        if (__ballot((o.a1 != kOutOfRange) | (o.b1 != kOutOfRange)) != 0ull) {
+          // (no streaming hint: a statistics row can be as small as 8 bytes, and the rows of the
+          // cp senders share 64-byte sectors that the L2 should merge before they go to memory)
+          __builtin_amdgcn_raw_buffer_store_b64(wa, st.field1, o.a1, 0, kAuxNone);
+          __builtin_amdgcn_raw_buffer_store_b64(wb, st.field1, o.b1, 0, kAuxNone);
+        }
       }
     }
   }
+  HELIX_MARK(wave, 2, false);
   if (lane == 0) {  // close the last entry (csrc/helix_alltoall.cu:468-472)
-    st_counter(&info[1], step + 1);
-    st_counter(&senderInfo[1], step + 1);
+    st_counter(mine, step + 1);
+    if (part == 0) st_counter(&senderInfo[1], step + 1);
   }
+  HELIX_MARK(wave, 3, true);
 }
 
 // The one wave-uniform branch on the units-in-flight count of the launch.
 template <int kAux>
-__device__ __forceinline__ void run_sender_any(const KernelArgs& a, int s, int r, int ch, int lane) {
+__device__ __forceinline__ void run_sender_any(const KernelArgs& a, int s, int r, int ch, int part, int lane, int wave) {
   switch (a.unitsInFlight) {
-    case 1: run_sender<kAux, 1>(a, s, r, ch, lane); break;
-    case 2: run_sender<kAux, 2>(a, s, r, ch, lane); break;
-    case 3: run_sender<kAux, 3>(a, s, r, ch, lane); break;
-    case 4: run_sender<kAux, 4>(a, s, r, ch, lane); break;
-    case 5: run_sender<kAux, 5>(a, s, r, ch, lane); break;
-    default: run_sender<kAux, kMaxUnitsInFlight>(a, s, r, ch, lane); break;
+    case 1: run_sender<kAux, 1>(a, s, r, ch, part, lane, wave); break;
+    case 2: run_sender<kAux, 2>(a, s, r, ch, part, lane, wave); break;
+    case 3: run_sender<kAux, 3>(a, s, r, ch, part, lane, wave); break;
+    case 4: run_sender<kAux, 4>(a, s, r, ch, part, lane, wave); break;
+    case 5: run_sender<kAux, 5>(a, s, r, ch, part, lane, wave); break;
+    default: run_sender<kAux, kMaxUnitsInFlight>(a, s, r, ch, part, lane, wave); break;
   }
 }
 // Wavefront w of a launch: sender wavefronts come first in dispatch order so
 // that no receiver can occupy a slot a not-yet-started sender needs.
-// Within a direction, w = (local rank * runChannels + channel) * cp + peer:
-// neighbouring wavefronts touch neighbouring rows of the same entry.
+// Within a direction, w = ((local rank * runChannels + channel) * cp + peer) * parts + part:
+// neighbouring wavefronts touch neighbouring slices, then neighbouring rows of the same entry.
 template <int kUnitsInFlight, bool kAlignedStores>
 __global__ __launch_bounds__(kBlockThreads) HELIX_WAVES_PER_SIMD void helix_exchange_kernel(KernelArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWaveLanes);
   const int lane = static_cast<int>(threadIdx.x) % kWaveLanes;
   int w = static_cast<int>(blockIdx.x) * kWavesPerBlock + wave;
-  const int perDirection = a.rankCount * a.runChannels * a.cpSize;
+  const int probe = w;  // index of this wavefront's phase stamps (a stamped build only)
+  const int perDirection = a.rankCount * a.runChannels * a.cpSize * a.parts;
   const int senders = a.doSend ? perDirection : 0;
   const int total = senders + (a.doRecv ? perDirection : 0);
   if (w >= total) return;
   const bool isSender = w < senders;
   if (!isSender) w -= senders;
-  const int peer = w % a.cpSize;
-  const int t = w / a.cpSize;
+  const int part = w % a.parts;
+  const int q = w / a.parts;
+  const int peer = q % a.cpSize;
+  const int t = q / a.cpSize;
   const int ch = t % a.runChannels;
   const int local = a.rankBegin + t / a.runChannels;
   if (isSender) {
-    run_sender<kAuxSc1, kUnitsInFlight>(a, local, peer, ch, lane);
+    run_sender<kAuxSc1, kUnitsInFlight>(a, local, peer, ch, part, lane, probe);
   } else {
-    run_receiver<kAuxSc1, kUnitsInFlight, kAlignedStores>(a, local, peer, ch, lane);
+    run_receiver<kAuxSc1, kUnitsInFlight, kAlignedStores>(a, local, peer, ch, part, lane, probe);
   }
 }
 
@@ -570,7 +593,8 @@ __device__ __forceinline__ u32x2 narrow_piece(const float (&acc)[4]) {
 
 template <int kDtype, int kLanesPerSlot>
 __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r, int ch, int part, int parts,
-                                                     int lane, CombineLds<kLanesPerSlot>& lds) {
+                                                     int lane, CombineLds<kLanesPerSlot>& lds, int probe) {
+  HELIX_MARK(probe, 0, false);
   constexpr int kSlotsPerPass = kWaveLanes / kLanesPerSlot;
   Stream st;
   setup_stream(st, a, 0, ch);
@@ -625,6 +649,7 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
       }
       asm volatile("" ::: "memory");
     }
+    if (firstMsg == 0) HELIX_MARK(probe, 1, false);
     for (uint32_t U0 = static_cast<uint32_t>(part) * kWaveLanes; U0 < runUnits;
          U0 += static_cast<uint32_t>(parts) * kWaveLanes) {
       const uint32_t U = U0 + lane;
@@ -765,6 +790,8 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
       __builtin_amdgcn_wave_barrier();  // the tables are rewritten by the next access
     }
   }
+  HELIX_MARK(probe, 2, false);
+  HELIX_MARK(probe, 3, true);
 }
 
 // Workgroups of `parts` wavefronts (blockDim.x / 64). The first
@@ -783,13 +810,36 @@ __global__ __launch_bounds__(kMaxCombineParts * kWaveLanes) HELIX_WAVES_PER_SIMD
     const int w = b * parts + wave;
     if (w >= senderStreams) return;
     const int t = w / a.cpSize;
-    run_sender_any<kAuxSc1>(a, a.rankBegin + t / a.runChannels, w % a.cpSize, t % a.runChannels, lane);
+    run_sender_any<kAuxSc1>(a, a.rankBegin + t / a.runChannels, w % a.cpSize, t % a.runChannels, 0, lane, w);
     return;
   }
   b -= sendBlocks;
   const int r = a.rankBegin + b / a.runChannels;
   const int ch = b % a.runChannels;
-  run_combine_receiver<kDtype, kLanesPerSlot>(a, r, ch, wave, parts, lane, lds);
+  run_combine_receiver<kDtype, kLanesPerSlot>(a, r, ch, wave, parts, lane, lds, senderStreams + b * parts + wave);
+}
+
+// Before a launch that shares runs between wavefronts: the step counters of parts 1.. of every stream
+// the launch touches take the value of part 0's (head on the sending side, tail on the receiving
+// side). Launches with one wavefront per stream move part 0's counters only, so the others may be
+// behind; this brings them level. One thread per (local rank, channel, peer) and direction.
+__global__ __launch_bounds__(256) void helix_level_part_counters_kernel(KernelArgs a) {
+  const int perDirection = a.rankCount * a.runChannels * a.cpSize;
+  int i = static_cast<int>(blockIdx.x * blockDim.x + threadIdx.x);
+  const int senders = a.doSend ? perDirection : 0;
+  const int total = senders + (a.doRecv ? perDirection : 0);
+  if (i >= total) return;
+  const bool sending = i < senders;
+  if (!sending) i -= senders;
+  const int peer = i % a.cpSize;
+  const int t = i / a.cpSize;
+  const int ch = t % a.runChannels;
+  const int local = a.rankBegin + t / a.runChannels;
+  uint8_t* row = a.workspace + static_cast<uint64_t>(local) * a.rowStrideBytes;
+  int64_t* info = reinterpret_cast<int64_t*>(
+      row + (sending ? sender_info_offset(a.cpSize, a.maxChannels, peer, ch) : receiver_info_offset(a.cpSize, a.maxChannels, peer, ch)));
+  const int64_t v = sending ? info[0] : info[1];
+  for (int p = 1; p < a.parts; ++p) info[sending ? sender_counter_slot(p) : receiver_counter_slot(p)] = v;
 }
 
 // FIFO region <- 0xFF bytes, info regions <- 0 (csrc/helix_alltoall.cu:637-643).
@@ -805,25 +855,31 @@ __global__ __launch_bounds__(256) void helix_init_row_kernel(u32x4* row, uint64_
 }  // namespace
 
 // The largest run of the launch is the first one of channel 0's streams.
-static KernelArgs with_units_in_flight(KernelArgs a) {
+static long largest_run_units(const KernelArgs& a) {
   const MsgShape sh = make_msg_shape(a.field0Bytes, a.field1Bytes);
   const int msgs = stream_msg_count(a.entryBegin, a.entryEnd, 0, a.runChannels);
   const int perEntry = msgs_per_fifo_entry(sh);
-  const long runUnits = run_units(msgs < perEntry ? msgs : perEntry, sh);
-  a.unitsInFlight = units_in_flight_for_run(runUnits);
-  a.alignedStores = runUnits > static_cast<long>(kMaxUnitsInFlight) * kWaveLanes ? 1 : 0;
-  return a;
+  return run_units(msgs < perEntry ? msgs : perEntry, sh);
 }
 
-hipError_t launch_exchange(const KernelArgs& args, hipStream_t stream) {
-  const KernelArgs a = with_units_in_flight(args);
+hipError_t launch_exchange(const KernelArgs& args, int unitsPerPart, int maxParts, hipStream_t stream) {
+  KernelArgs a = args;
+  const long runUnits = largest_run_units(a);
+  const RunSplit split = split_for_run(runUnits, unitsPerPart, maxParts);
+  a.parts = split.parts;
+  a.unitsInFlight = split.unitsInFlight;
+  a.alignedStores = runUnits > static_cast<long>(kMaxUnitsInFlight) * kWaveLanes ? 1 : 0;
   int directions = (a.doSend ? 1 : 0) + (a.doRecv ? 1 : 0);
-  int waves = directions * waves_per_direction(a);
+  int waves = directions * waves_per_direction(a) * a.parts;
   if (waves <= 0) return hipSuccess;
+  if (a.parts > 1) {
+    const int threads = directions * waves_per_direction(a);
+    hipLaunchKernelGGL(helix_level_part_counters_kernel, dim3((threads + 255) / 256), dim3(256), 0, stream, a);
+  }
   int blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
-  // Runs of one pass: 1..6 units in flight, payload stored piece by piece. Runs of
-  // several passes (at least 4 units in flight by the rule): the instantiation
-  // whose receivers realign the payload to 16-byte stores.
+  // Short runs: 1..6 units in flight, payload stored piece by piece. Long runs (more than one
+  // pass of six; at least 4 units in flight by the rule): the instantiation whose receivers
+  // realign the payload to 16-byte stores.
 #define HELIX_LAUNCH_EXCHANGE(K, ALIGNED) \
   hipLaunchKernelGGL((helix_exchange_kernel<K, ALIGNED>), dim3(blocks), dim3(kBlockThreads), 0, stream, a)
   if (a.alignedStores && a.unitsInFlight >= 4) {
@@ -847,7 +903,9 @@ hipError_t launch_exchange(const KernelArgs& args, hipStream_t stream) {
 }
 
 hipError_t launch_combine(const KernelArgs& args, int parts, hipStream_t stream) {
-  const KernelArgs a = with_units_in_flight(args);
+  KernelArgs a = args;
+  a.parts = 1;  // the senders of this kernel walk whole runs
+  a.unitsInFlight = units_in_flight_for_run(largest_run_units(a));
   const int senderStreams = a.doSend ? a.rankCount * a.runChannels * a.cpSize : 0;
   if (a.rankCount * a.runChannels <= 0) return hipSuccess;
   if (parts < 1) parts = 1;
@@ -871,6 +929,20 @@ hipError_t launch_combine(const KernelArgs& args, int parts, hipStream_t stream)
 #undef HELIX_LAUNCH_COMBINE
   return hipGetLastError();
 }
+
+#ifdef HELIX_A2A_TIMELINE
+// Copies the phase stamps of the first `waves` wavefronts of the launches so far to the host
+// (four 100 MHz clock values per wavefront) and clears them. Stamped builds only.
+extern "C" int helix_a2a_timeline_read(uint64_t* host, int waves) {
+  if (waves < 0 || waves > kTimelineWaves) return 1;
+  void* dev = nullptr;
+  if (hipGetSymbolAddress(&dev, HIP_SYMBOL(g_timeline)) != hipSuccess) return 2;
+  if (hipDeviceSynchronize() != hipSuccess) return 2;
+  if (hipMemcpy(host, dev, static_cast<size_t>(waves) * 4 * sizeof(uint64_t), hipMemcpyDeviceToHost) != hipSuccess) return 2;
+  if (hipMemset(dev, 0, static_cast<size_t>(kTimelineWaves) * 4 * sizeof(uint64_t)) != hipSuccess) return 2;
+  return 0;
+}
+#endif
 
 hipError_t launch_init_row(uint8_t* row, uint64_t fifoBytes, uint64_t infoBytes, hipStream_t stream) {
   uint64_t fifoUnits = fifoBytes / kUnitBytes;

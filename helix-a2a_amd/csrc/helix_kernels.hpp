@@ -37,6 +37,7 @@ struct KernelArgs {
   int doSend, doRecv;
   int unitsInFlight;        // units_in_flight_for_run(largest run of the launch), 1..kMaxUnitsInFlight
   int alignedStores;        // receivers realign payload to 16-byte stores: set when runs take several passes
+  int parts;                // wavefronts that share one stream's runs (per direction), 1..kMaxStreamParts
   uint64_t spinLimitTicks;  // bound of one in-kernel wait, in 100 MHz ticks
   uint32_t* status;         // device status word (HELIX_A2A_STATUS_* bits)
   // combine only
@@ -50,10 +51,12 @@ struct KernelArgs {
 constexpr int kWavesPerBlock = 2;
 constexpr int kBlockThreads = kWavesPerBlock * kWaveLanes;
 
-// wavefronts one direction of a launch needs: one per (local rank, channel, peer)
+// streams one direction of a launch serves: one per (local rank, channel, peer)
 inline int waves_per_direction(const KernelArgs& a) { return a.rankCount * a.runChannels * a.cpSize; }
 
-hipError_t launch_exchange(const KernelArgs& a, hipStream_t stream);
+// A stream's runs are shared by as many wavefronts (at most maxParts) as leave each at most
+// unitsPerPart units per lane; maxParts = 1: one wavefront per stream.
+hipError_t launch_exchange(const KernelArgs& a, int unitsPerPart, int maxParts, hipStream_t stream);
 // exchange fused with the LSE-weighted combine, all ranks of the launch; `parts` wavefronts share
 // the units of one (receiver, channel)
 constexpr int kMaxCombineParts = 8;

@@ -193,4 +193,75 @@ HELIX_HD int units_in_flight_for_run(long runUnits) {
   return static_cast<int>((perLane + passes - 1) / passes);
 }
 
+
+// ---- runs shared by several wavefronts ---------------------------------------
+// A long run can be cut into `parts` slices of whole wave accesses (64 units),
+// one wavefront per slice and direction. A launch that would leave most of the
+// device idle (few streams, long runs) is spread over more wavefronts that way;
+// a launch that fills the device anyway is not split (measured on MI355X: more,
+// shorter wavefronts for the same bytes are slower once every slot is taken).
+//
+// Every part of a stream keeps a step counter of its own in the stream's
+// 256-byte counter blocks (32 slots of 8 bytes; the reference uses two,
+// csrc/helix_alltoall.cu:61-64): part 0 uses the reference's head (sender
+// block, slot 0) and tail (receiver block, slot 1; its copy for the sender's
+// back-pressure in the sender block, slot 1), part p >= 1 uses slot p + 1 of
+// either block. A sender part moves its counter beyond a step once its stores
+// of that step are acknowledged: that is the token its receiver part waits for.
+// A launch moves the counters of the parts it has; a launch with more than one
+// part first brings the counters of its parts 1.. level with part 0's, so
+// launches may differ in their number of parts.
+constexpr int kCounterSlots = kFifoInfoBytes / 8;     // 32
+constexpr int kMaxStreamParts = 16;
+HELIX_HD int sender_counter_slot(int part) { return part == 0 ? 0 : part + 1; }
+HELIX_HD int receiver_counter_slot(int part) { return part + 1; }
+
+struct RunSplit {
+  int parts;          // wavefronts per stream and direction
+  int unitsInFlight;  // units a lane keeps in flight per pass over its slice
+};
+// For the largest run of a launch: as many parts (at most maxParts, at most kMaxStreamParts) as leave each
+// at most unitsPerPart units per lane; then the slice of a part in the fewest passes of at most
+// kMaxUnitsInFlight units per lane, with the smallest count that still makes that number of passes.
+HELIX_HD RunSplit split_for_run(long runUnits, int unitsPerPart, int maxParts) {
+  if (unitsPerPart < 1) unitsPerPart = 1;
+  if (unitsPerPart > kMaxUnitsInFlight) unitsPerPart = kMaxUnitsInFlight;
+  if (maxParts > kMaxStreamParts) maxParts = kMaxStreamParts;
+  if (maxParts < 1) maxParts = 1;
+  long perLane = (runUnits + kWaveLanes - 1) / kWaveLanes;
+  if (perLane < 1) perLane = 1;
+  long parts = (perLane + unitsPerPart - 1) / unitsPerPart;
+  if (parts > maxParts) parts = maxParts;
+  long slicePerLane = (perLane + parts - 1) / parts;
+  long passes = (slicePerLane + kMaxUnitsInFlight - 1) / kMaxUnitsInFlight;
+  RunSplit r;
+  r.parts = static_cast<int>(parts);
+  r.unitsInFlight = static_cast<int>((slicePerLane + passes - 1) / passes);
+  return r;
+}
+// Wavefronts per stream the automatic rule allows: as many as the wavefront slots of the device (four per
+// SIMD, sixteen per compute unit) leave room for when every stream of the exchange -- both directions of
+// all cp ranks, whatever part of it a launch carries -- takes that many.
+HELIX_HD int auto_max_parts(int cpSize, int runChannels, int cuCount) {
+  const long slots = static_cast<long>(cuCount) * 16;
+  const long streams = 2L * cpSize * cpSize * runChannels;
+  const long parts = streams > 0 ? slots / streams : 1;
+  return parts < 1 ? 1 : (parts > kMaxStreamParts ? kMaxStreamParts : static_cast<int>(parts));
+}
+
+// units [begin, end) of a run of `runUnits` units that part `part` of `parts` walks
+struct Slice {
+  uint32_t begin, end;
+};
+HELIX_HD Slice slice_of_run(uint32_t runUnits, int part, int parts) {
+  const uint32_t perLane = (runUnits + kWaveLanes - 1) / kWaveLanes;
+  const uint32_t slice = (perLane + parts - 1) / parts * kWaveLanes;
+  Slice s;
+  s.begin = static_cast<uint32_t>(part) * slice;
+  if (s.begin > runUnits) s.begin = runUnits;
+  s.end = s.begin + slice;
+  if (s.end > runUnits) s.end = runUnits;
+  return s;
+}
+
 }  // namespace helix

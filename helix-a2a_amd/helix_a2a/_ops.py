@@ -79,6 +79,8 @@ def _load_library() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.argtypes = [P(_Params), ctypes.c_int, ctypes.c_void_p]
         fn.restype = ctypes.c_int
+    lib.helix_a2a_set_units_per_wavefront.argtypes = [ctypes.c_int]
+    lib.helix_a2a_set_units_per_wavefront.restype = ctypes.c_int
     lib.helix_a2a_alltoall_combine_loopback.argtypes = [
         P(_Params), P(_CombineOut), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
     lib.helix_a2a_alltoall_combine_loopback.restype = ctypes.c_int
@@ -235,12 +237,13 @@ def _make_params(o3: torch.Tensor, s3: torch.Tensor, out_o: Optional[torch.Tenso
     if out_s is not None:
         _fill_field(p.recv_fields[1], out_s)
     p.entry_count = o3.size(0)
-    p.workspace = workspace.data_ptr()
-    p.workspace_stride_u64 = workspace.stride(0)
     p.cp_rank = cp_rank
     p.cp_size = cp_size
     p.channel_count = int(channel_count)
-    p.max_channel_count = max_channel_count(cp_size)
+    if workspace is not None:
+        p.workspace = workspace.data_ptr()
+        p.workspace_stride_u64 = workspace.stride(0)
+        p.max_channel_count = max_channel_count(cp_size)
     return p
 
 
@@ -569,6 +572,11 @@ def device_status() -> int:
 
 def set_spin_limit_us(microseconds: int) -> None:
     _lib.helix_a2a_set_spin_limit_us(int(microseconds))
+
+
+def set_units_per_wavefront(units: int) -> None:
+    """Share a stream's runs longer than ``units`` KiB between wavefronts: 1..6 always, 0 never, -1 (default) beyond 6 KiB while the launch leaves the device under-filled."""
+    _check(_lib.helix_a2a_set_units_per_wavefront(int(units)), "set_units_per_wavefront")
 
 
 def set_single_round(enabled: bool) -> None:

@@ -208,6 +208,25 @@ void helix_a2a_set_spin_limit_us(uint64_t microseconds);
  */
 void helix_a2a_set_single_round(int enabled);
 
+/*
+ * How much of a stream's run one wavefront takes (process-wide; takes effect
+ * with the next call). A run can be shared by up to 16 wavefronts per
+ * direction, each with a step counter of its own in the stream's counter
+ * blocks.
+ *   -1 (default)  share runs longer than 6 units per lane (6 KiB), but only
+ *                 while the launch leaves wavefront slots of the device free:
+ *                 few streams with long runs are spread over the device, a
+ *                 launch that fills it anyway is left alone
+ *    0            never: one wavefront per stream however long its runs (the
+ *                 reference's shape, one warp per stream,
+ *                 csrc/helix_alltoall.cu:315-330)
+ *    1..6         always share runs longer than that many units per lane
+ * The send and the receive half of one exchange must run under the same
+ * setting. No counterpart in the reference. Returns 0 or
+ * HELIX_A2A_ERR_INVALID_ARGUMENT.
+ */
+int helix_a2a_set_units_per_wavefront(int units);
+
 /* thread-local message of the most recent failure on this thread ("" if none) */
 const char* helix_a2a_last_error(void);
 

@@ -60,6 +60,10 @@ class HostModel:
         lib.hm_unit_first_piece.restype = ctypes.c_int
         lib.hm_units_in_flight.argtypes = [ctypes.c_long]
         lib.hm_units_in_flight.restype = ctypes.c_int
+        lib.hm_split_for_run.argtypes = [ctypes.c_long, ctypes.c_int, ctypes.c_int]
+        lib.hm_split_for_run.restype = ctypes.c_int
+        lib.hm_set_units_per_part.argtypes = [ctypes.c_int]
+        lib.hm_set_units_per_part.restype = None
         lib.hm_div.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
         lib.hm_div.restype = ctypes.c_uint32
         lib.hm_div_mismatches.argtypes = [ctypes.c_uint32]
@@ -69,6 +73,15 @@ class HostModel:
         lib.hm_msgs_per_entry.argtypes = [ctypes.c_int] * 2
         lib.hm_msgs_per_entry.restype = ctypes.c_int
         self.lib = lib
+
+    def split_for_run(self, run_units: int, units_per_part: int = 6, max_parts: int = 16) -> Tuple[int, int]:
+        """(wavefronts per stream, units in flight) the launch rule picks for a largest run of ``run_units`` units."""
+        v = self.lib.hm_split_for_run(run_units, units_per_part, max_parts)
+        return v >> 8, v & 255
+
+    def set_units_per_part(self, units: int) -> None:
+        """The library's knob: -1 automatic (default), 0 one wavefront per stream, 1..6 share runs longer than that."""
+        self.lib.hm_set_units_per_part(units)
 
     @staticmethod
     def max_channel_count(cp: int, cu_count: int) -> int:

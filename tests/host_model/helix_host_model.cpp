@@ -49,8 +49,11 @@ struct Ctx {
   Extent ws;
   Checker chk;
   int unitsInFlight;   // per round, by the library's rule
-  bool alignedStores;  // receivers of multi-pass runs store realigned 16-byte pieces
+  int parts;           // wavefronts that share a stream's runs, by the library's rule
+  bool alignedStores;  // receivers of long runs store realigned 16-byte pieces
 };
+
+int g_unitsPerPart = -1;  // the library's knob: -1 automatic, 0 one wavefront per stream, 1..6 share runs longer than that per lane
 
 Extent field_extent(const helix_a2a_field_t& f, int entries, int cp) {
   return Extent{static_cast<const uint8_t*>(f.data), static_cast<uint64_t>(entries) * cp * f.stride_bytes};
@@ -82,8 +85,8 @@ UnitOffsets unit_offsets(const Ctx& c, uint32_t firstRow, uint32_t rowStep, uint
   return o;
 }
 
-// sender wave of stream (s -> r, ch): one run per FIFO entry, units walked flat
-void run_sender(Ctx& c, int s, int r, int ch) {
+// part `part` of the sender waves of stream (s -> r, ch): one run per FIFO entry, its slice of the units walked flat
+void run_sender(Ctx& c, int s, int r, int ch, int part) {
   const helix_a2a_params_t& p = c.ranks[s];
   uint8_t* wsBase = reinterpret_cast<uint8_t*>(p.workspace);
   uint64_t rowStride = p.workspace_stride_u64 * 8;
@@ -91,7 +94,8 @@ void run_sender(Ctx& c, int s, int r, int ch) {
   uint8_t* receiverRow = wsBase + r * rowStride;
   int64_t* info = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(c.cp, c.maxCh, r, ch));
   uint8_t* fifo = receiverRow + fifo_offset(s, ch, c.maxCh);
-  if (!c.chk.ok(c.ws, info, 16, "sender info") || !c.chk.ok(c.ws, fifo, kFifoBytes, "fifo")) return;
+  if (!c.chk.ok(c.ws, info, kFifoInfoBytes, "sender info") || !c.chk.ok(c.ws, fifo, kFifoBytes, "fifo")) return;
+  int64_t* token = info + sender_counter_slot(part);
   Extent fifoExt{fifo, kFifoBytes};
   Extent e0 = field_extent(p.send_fields[0], p.entry_count, c.cp);
   Extent e1 = field_extent(p.send_fields[1], p.entry_count, c.cp);
@@ -100,13 +104,14 @@ void run_sender(Ctx& c, int s, int r, int ch) {
   const int perEntry = msgs_per_fifo_entry(c.sh);
   const uint32_t firstRow = static_cast<uint32_t>(c.entryBegin + ch) * c.cp + r;
   const uint32_t rowStep = static_cast<uint32_t>(c.channels) * c.cp;
-  int64_t step = info[0];
+  int64_t step = *token;
   for (int firstMsg = 0; firstMsg < msgs; firstMsg += perEntry) {
     int runMsgs = perEntry < msgs - firstMsg ? perEntry : msgs - firstMsg;
     uint32_t runUnits = static_cast<uint32_t>(run_units(runMsgs, c.sh));
+    const Slice slice = slice_of_run(runUnits, part, c.parts);
     if (firstMsg > 0) {
       step += 1;
-      info[0] = step;
+      *token = step;
     }
     // the model runs senders to completion first: room must already be there
     if (info[1] + kFifoDepth <= step) {
@@ -116,7 +121,7 @@ void run_sender(Ctx& c, int s, int r, int ch) {
       return;
     }
     uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
-    for (uint32_t U = 0; U < runUnits; ++U) {  // every lane of every wave access
+    for (uint32_t U = slice.begin; U < slice.end; ++U) {  // every lane of every wave access
       UnitOffsets o = unit_offsets(c, firstRow, rowStep, p.send_fields[0].stride_bytes, p.send_fields[1].stride_bytes,
                                    firstMsg, runMsgs, U);
       uint64_t words[2] = {0, 0};
@@ -130,11 +135,12 @@ void run_sender(Ctx& c, int s, int r, int ch) {
       if (c.chk.ok(fifoExt, dst, 16, "fifo store")) memcpy(dst, words, 16);
     }
   }
-  info[0] = step + 1;
+  *token = step + 1;
 }
 
-// receiver wave of stream (s -> r, ch); a line whose flag is not there counts as a violation
-void run_receiver(Ctx& c, int r, int s, int ch) {
+// part `part` of the receiver waves of stream (s -> r, ch); a missing token or a line whose flag is not there
+// counts as a violation
+void run_receiver(Ctx& c, int r, int s, int ch, int part) {
   const helix_a2a_params_t& p = c.ranks[r];
   uint8_t* wsBase = reinterpret_cast<uint8_t*>(p.workspace);
   uint64_t rowStride = p.workspace_stride_u64 * 8;
@@ -143,9 +149,11 @@ void run_receiver(Ctx& c, int r, int s, int ch) {
   int64_t* sinfo = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(c.cp, c.maxCh, r, ch));
   int64_t* info = reinterpret_cast<int64_t*>(receiverRow + receiver_info_offset(c.cp, c.maxCh, s, ch));
   uint8_t* fifo = receiverRow + fifo_offset(s, ch, c.maxCh);
-  if (!c.chk.ok(c.ws, info, 16, "receiver info") || !c.chk.ok(c.ws, sinfo, 16, "sender info") ||
+  if (!c.chk.ok(c.ws, info, kFifoInfoBytes, "receiver info") || !c.chk.ok(c.ws, sinfo, kFifoInfoBytes, "sender info") ||
       !c.chk.ok(c.ws, fifo, kFifoBytes, "fifo"))
     return;
+  const int64_t* token = sinfo + sender_counter_slot(part);
+  int64_t* mine = info + receiver_counter_slot(part);
   Extent fifoExt{fifo, kFifoBytes};
   Extent e0 = field_extent(p.recv_fields[0], p.entry_count, c.cp);
   Extent e1 = field_extent(p.recv_fields[1], p.entry_count, c.cp);
@@ -154,14 +162,21 @@ void run_receiver(Ctx& c, int r, int s, int ch) {
   const int perEntry = msgs_per_fifo_entry(c.sh);
   const uint32_t firstRow = static_cast<uint32_t>(c.entryBegin + ch) * c.cp + s;
   const uint32_t rowStep = static_cast<uint32_t>(c.channels) * c.cp;
-  int64_t step = info[1];
+  int64_t step = *mine;
   for (int firstMsg = 0; firstMsg < msgs; firstMsg += perEntry) {
     int runMsgs = perEntry < msgs - firstMsg ? perEntry : msgs - firstMsg;
     uint32_t runUnits = static_cast<uint32_t>(run_units(runMsgs, c.sh));
+    const Slice slice = slice_of_run(runUnits, part, c.parts);
     if (firstMsg > 0) {
       step += 1;
-      info[1] = step;
-      sinfo[1] = step;
+      *mine = step;
+      if (part == 0) sinfo[1] = step;
+    }
+    if (*token <= step) {  // the sending part has not closed this step: the GPU receiver would wait here
+      if (c.chk.violations++ == 0)
+        snprintf(c.chk.first, sizeof(c.chk.first), "stream %d->%d ch %d part %d: token %lld not beyond step %lld", s, r, ch,
+                 part, (long long)*token, (long long)step);
+      return;
     }
     uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
     uint8_t* base0 = const_cast<uint8_t*>(e0.base);
@@ -169,7 +184,8 @@ void run_receiver(Ctx& c, int r, int s, int ch) {
     const uint32_t stride0 = p.recv_fields[0].stride_bytes, stride1 = p.recv_fields[1].stride_bytes;
     // one pass = unitsInFlight accesses of 64 lanes, all loaded before anything is stored
     const uint32_t passUnits = static_cast<uint32_t>(c.unitsInFlight) * kWaveLanes;
-    for (uint32_t U0 = 0; U0 < runUnits; U0 += passUnits) {
+    for (uint32_t U0 = slice.begin; U0 < slice.end; U0 += passUnits) {
+      const uint32_t passEnd = U0 + passUnits < slice.end ? U0 + passUnits : slice.end;
       uint64_t words[kMaxUnitsInFlight][kWaveLanes][2];
       bool landed[kMaxUnitsInFlight][kWaveLanes];
       for (int i = 0; i < c.unitsInFlight; ++i) {
@@ -177,7 +193,7 @@ void run_receiver(Ctx& c, int r, int s, int ch) {
           const uint32_t U = U0 + i * kWaveLanes + lane;
           landed[i][lane] = false;
           words[i][lane][0] = words[i][lane][1] = 0;  // what an out-of-range load returns
-          if (U >= runUnits) continue;
+          if (U >= passEnd) continue;
           const uint8_t* src = fifo + entryOffset + U * kUnitBytes;
           if (!c.chk.ok(fifoExt, src, 16, "fifo load")) continue;
           memcpy(words[i][lane], src, 16);
@@ -201,8 +217,8 @@ void run_receiver(Ctx& c, int r, int s, int ch) {
           const uint64_t* w = words[i][lane];
           if (c.alignedStores) {
             // the aligned 16 bytes that start at whichever word is an even partial_o piece; second half from the next unit
-            const bool haveNext = lane < kWaveLanes - 1 || i + 1 < c.unitsInFlight;
-            const uint64_t nextFirst = lane < kWaveLanes - 1 ? words[i][lane + 1][0] : (haveNext ? words[i + 1][0][0] : 0);
+            const bool haveNext = U + 1 < passEnd;
+            const uint64_t nextFirst = lane < kWaveLanes - 1 ? words[i][lane + 1][0] : (i + 1 < c.unitsInFlight ? words[i + 1][0][0] : 0);
             const bool startsAtA = o.a0 != kNone && (d.pieceA & 1u) == 0;
             const bool startsAtB = o.b0 != kNone && (d.pieceB & 1u) == 0;
             const bool takesNext = startsAtB || (startsAtA && d.flag);
@@ -211,8 +227,7 @@ void run_receiver(Ctx& c, int r, int s, int ch) {
               uint8_t* dst = base0 + (startsAtB ? o.b0 : o.a0);
               if (c.chk.ok(e0, dst, 16, "recv field 0 (16 bytes)")) memcpy(dst, chunk, 16);
             }
-            const bool alone = o.a0 != kNone && ((i == c.unitsInFlight - 1 && lane == kWaveLanes - 1 && startsAtA && d.flag) ||
-                                                 (i == 0 && lane == 0 && (d.pieceA & 1u) != 0));
+            const bool alone = o.a0 != kNone && ((U + 1 == passEnd && startsAtA && d.flag) || (U == U0 && (d.pieceA & 1u) != 0));
             if (alone) {
               uint8_t* dst = base0 + o.a0;
               if (c.chk.ok(e0, dst, 8, "recv field 0 (lone piece)")) memcpy(dst, &w[0], 8);
@@ -229,8 +244,25 @@ void run_receiver(Ctx& c, int r, int s, int ch) {
       }
     }
   }
-  info[1] = step + 1;
-  sinfo[1] = step + 1;
+  *mine = step + 1;
+  if (part == 0) sinfo[1] = step + 1;
+}
+
+// what the library does ahead of a launch that shares runs between wavefronts: the counters of
+// parts 1.. of every stream of the launch take the value of part 0's
+void level_part_counters(Ctx& c, bool send, bool recv) {
+  for (int local = 0; local < c.cp; ++local)
+    for (int ch = 0; ch < c.channels; ++ch)
+      for (int peer = 0; peer < c.cp; ++peer) {
+        uint8_t* row = reinterpret_cast<uint8_t*>(c.ranks[0].workspace) + local * c.ranks[0].workspace_stride_u64 * 8;
+        int64_t* si = reinterpret_cast<int64_t*>(row + sender_info_offset(c.cp, c.maxCh, peer, ch));
+        int64_t* ri = reinterpret_cast<int64_t*>(row + receiver_info_offset(c.cp, c.maxCh, peer, ch));
+        if (!c.chk.ok(c.ws, si, kFifoInfoBytes, "sender info") || !c.chk.ok(c.ws, ri, kFifoInfoBytes, "receiver info")) return;
+        for (int p = 1; p < c.parts; ++p) {
+          if (send) si[sender_counter_slot(p)] = si[0];
+          if (recv) ri[receiver_counter_slot(p)] = ri[1];
+        }
+      }
 }
 
 }  // namespace
@@ -270,21 +302,36 @@ int hm_alltoall(const helix_a2a_params_t* per_rank, int cp, int cu_count, int ch
       const int msgs0 = stream_msg_count(c.entryBegin, c.entryEnd, 0, channels);
       const int perEntry = msgs_per_fifo_entry(c.sh);
       const long maxRun = run_units(msgs0 < perEntry ? msgs0 : perEntry, c.sh);
-      c.unitsInFlight = units_in_flight_for_run(maxRun);
+      const RunSplit split = g_unitsPerPart == 0  ? split_for_run(maxRun, kMaxUnitsInFlight, 1)
+                             : g_unitsPerPart > 0 ? split_for_run(maxRun, g_unitsPerPart, kMaxStreamParts)
+                                                  : split_for_run(maxRun, kMaxUnitsInFlight, auto_max_parts(cp, channels, cu_count));
+      c.parts = split.parts;
+      c.unitsInFlight = split.unitsInFlight;
       c.alignedStores = maxRun > static_cast<long>(kMaxUnitsInFlight) * kWaveLanes;
     }
+    if (c.parts > 1) level_part_counters(c, do_send != 0, do_recv != 0);
     if (do_send)
       for (int s = 0; s < cp; ++s)
         for (int ch = 0; ch < channels; ++ch)
-          for (int r = 0; r < cp; ++r) run_sender(c, s, r, ch);
+          for (int r = 0; r < cp; ++r)
+            for (int part = 0; part < c.parts; ++part) run_sender(c, s, r, ch, part);
     if (do_recv)
       for (int r = 0; r < cp; ++r)
         for (int ch = 0; ch < channels; ++ch)
-          for (int s = 0; s < cp; ++s) run_receiver(c, r, s, ch);
+          for (int s = 0; s < cp; ++s)
+            for (int part = 0; part < c.parts; ++part) run_receiver(c, r, s, ch, part);
   }
   if (c.chk.violations) snprintf(g_msg, sizeof(g_msg), "%s", c.chk.first);
   g_outOfExtent = c.chk.outOfExtent;
   return c.chk.violations;
+}
+
+// the library's knob (helix_a2a_set_units_per_wavefront): -1 automatic, 0 never share, 1..6 always beyond that
+void hm_set_units_per_part(int units) { g_unitsPerPart = units; }
+// what the launch rule makes of a largest run of `runUnits` units: parts * 256 + units in flight
+int hm_split_for_run(long runUnits, int unitsPerPart, int maxParts) {
+  const RunSplit r = split_for_run(runUnits, unitsPerPart, maxParts);
+  return r.parts * 256 + r.unitsInFlight;
 }
 
 // geometry probes for tests

@@ -328,6 +328,31 @@ def test_runs_of_several_passes(hx, ops, cp, entries, x, s, channels):
     check_against_oracle(ins_o, ins_s, outs_o, outs_s)
 
 
+@pytest.mark.parametrize("units", [0, 1, 2, 3, 4, 5])
+def test_runs_shared_by_several_wavefronts(hx, ops, units):
+    # every split of a stream's runs over wavefronts gives the same bits, on one workspace, call after call:
+    # the step counters of all parts of a stream move in lockstep whatever the number of parts of a call
+    shapes = [(3, 7, 1096, 6, 2), (8, 256, 1024, 16, 128), (2, 9, 61432, 2, 1), (4, 12, 1016, 14, 1), (16, 64, 264, 2, 4)]
+    try:
+        for cp, entries, x, s, channels in shapes:
+            ws = get_workspace(hx, cp)
+            g = torch.Generator().manual_seed(cp * 31 + entries + units)
+            ins_o = [torch.randint(-32768, 32767, (entries, cp, x), generator=g, dtype=torch.int16).view(torch.bfloat16).cuda()
+                     for _ in range(cp)]
+            ins_s = [torch.randint(-2**31, 2**31 - 1, (entries, cp, s), generator=g, dtype=torch.int32).view(torch.float32).cuda()
+                     for _ in range(cp)]
+            for u in (units, 6, units):
+                ops.set_units_per_wavefront(u)
+                outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws, channel_count=channels)
+                torch.cuda.synchronize()
+                assert_clean(ops)
+                check_against_oracle(ins_o, ins_s, outs_o, outs_s, with_numpy=False)
+    finally:
+        ops.set_units_per_wavefront(-1)
+    with pytest.raises(RuntimeError, match="units per wavefront"):
+        ops.set_units_per_wavefront(7)
+
+
 def test_special_values_survive(hx, ops):
     # NaN payloads, infinities, denormals and negative zero are bytes like any other
     cp, entries = 2, 4

@@ -203,12 +203,77 @@ def test_rounds_when_traffic_exceeds_the_fifo(host_model):
 
 
 def test_receiver_rejects_stale_lines(host_model):
-    # a receive without the matching send must find no valid flag (fresh FIFO holds all ones)
+    # a receive without the matching send finds no token (the sender's counter has not moved) ...
     cp = 2
     ins_o, ins_s = random_inputs(cp, 3, 64, 2, seed=2)
     ws = host_model.new_workspace(cp, CU)
     _, _, rc, msg = host_model.alltoall(ins_o, ins_s, ws, CU, 1, send=False, recv=True)
+    assert rc > 0 and "token" in msg
+    # ... and with a forged token, no valid flag: a fresh FIFO holds all ones
+    max_ch = host_model.max_channel_count(cp, CU)
+    for sender in range(cp):
+        for receiver in range(cp):
+            ws[sender][host_model.lib.hm_sender_info_offset(cp, max_ch, receiver, 0) // 8] = 1
+    _, _, rc, msg = host_model.alltoall(ins_o, ins_s, ws, CU, 1, send=False, recv=True)
     assert rc > 0 and "flag" in msg
+
+
+def test_split_rule(host_model):
+    # wavefronts per stream: as many as leave each at most `units per part` units per lane (16 at most);
+    # units in flight: the slice of a part in the fewest passes of at most 6, then the smallest such count
+    f = host_model.split_for_run
+    assert f(144) == (1, 3)      # c2's run: 18 lines
+    assert f(288) == (1, 5)      # c3: 36 lines, 4.5 units per lane
+    assert f(584) == (2, 5)      # c5a: 73 lines
+    assert f(1104) == (3, 6)     # c4: 138 lines
+    assert f(8192) == (16, 4)    # a full FIFO entry: 128 units per lane, 8 per part in two passes of 4
+    assert f(288, 3) == (2, 3)
+    assert f(0) == (1, 1)
+    assert f(8192, 6, 1) == (1, 6) and f(8192, 6, 4) == (4, 6) and f(1104, 6, 2) == (2, 5)
+    for units in range(0, 8193, 17):      # one wavefront per stream: the units-in-flight rule alone
+        assert f(units, 6, 1) == (1, host_model.lib.hm_units_in_flight(units))
+    for units in range(1, 8193, 13):
+        for per_part in (1, 2, 3, 4, 5, 6):
+            parts, k = f(units, per_part)
+            per_lane = -(-units // 64)
+            slice_per_lane = -(-per_lane // parts)
+            passes = -(-slice_per_lane // 6)
+            assert 1 <= parts <= 16 and 1 <= k <= 6
+            assert parts == min(-(-per_lane // per_part), 16)
+            assert k * passes >= slice_per_lane and (k - 1) * passes < slice_per_lane
+
+
+@pytest.mark.parametrize("units_per_part", [0, 1, 2, 3, 6])
+def test_runs_shared_by_several_wavefronts(host_model, units_per_part):
+    # the same exchange whatever the number of wavefronts per stream, also when calls on one workspace
+    # differ in it: a call brings the counters of its parts level before it starts
+    cp, entries, x, s = 3, 7, 1096, 6        # 277 pieces per message; channel 0 carries 4 messages = 74 lines
+    ins_o, ins_s = random_inputs(cp, entries, x, s, seed=11)
+    host_model.set_units_per_part(units_per_part)
+    try:
+        out_o, out_s, ws = _exchange(host_model, ins_o, ins_s, channels=2)
+        # a second call on the same workspace with the default split: counters of all parts are in step
+        host_model.set_units_per_part(6)
+        out_o2, out_s2, _ = _exchange(host_model, ins_o, ins_s, channels=2, ws=ws)
+    finally:
+        host_model.set_units_per_part(-1)
+    want_o, want_s = ho.exchange_closed_form(ins_o), ho.exchange_closed_form(ins_s)
+    for r in range(cp):
+        assert (out_o[r] == want_o[r]).all() and (out_s[r] == want_s[r]).all()
+        assert (out_o2[r] == want_o[r]).all() and (out_s2[r] == want_s[r]).all()
+    max_ch = host_model.max_channel_count(cp, CU)
+    parts = {0: 1, 1: 10, 2: 5, 3: 4, 6: 2}[units_per_part]      # 74 lines = 592 units = 10 units per lane
+    for a in range(cp):
+        for b in range(cp):
+            for ch in range(2):
+                so = host_model.lib.hm_sender_info_offset(cp, max_ch, b, ch) // 8
+                ro = host_model.lib.hm_receiver_info_offset(cp, max_ch, b, ch) // 8
+                # head and tail count both calls; so do the counters of the parts the second call had (two);
+                # parts only the first call had stay where that call left them
+                assert ws[a][so] == 2 and ws[a][so + 1] == 2 and ws[a][ro + 1] == 2 and ws[a][ro] == 0
+                for p in range(1, 16):
+                    want = 2 if p < 2 else (1 if p < parts else 0)
+                    assert ws[a][so + p + 1] == want and ws[a][ro + p + 1] == want, (p, parts)
 
 
 def test_bounds_checker_catches_short_buffers(host_model):
