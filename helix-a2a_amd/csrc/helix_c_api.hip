@@ -65,11 +65,22 @@ struct DeviceState {
   hipError_t initError = hipSuccess;
   int cuCount = 0;
   uint32_t* status = nullptr;  // device status word
+  uint8_t* scratch = nullptr;  // this device's copy of the built-in workspace (helix_a2a_alltoall_loopback_static)
+  std::mutex scratchMutex;
+  int scratchCp = 0;           // cp_size the built-in workspace is laid out and initialised for (0 = not yet)
 };
 DeviceState g_devices[kMaxDevices];
 
 // status word: one per device, lives until the process ends
 __device__ uint32_t g_statusWord[4];
+
+// Built-in workspace of helix_a2a_alltoall_loopback_static: room for kStaticStreams FIFOs
+// (sender, receiver, channel) with their two counter blocks, 64.06 MiB, held by every device the
+// library runs on until the process ends. In host code the name is only a handle for
+// hipGetSymbolAddress; kernels and fills get the per-device address kept in DeviceState::scratch.
+constexpr int kStaticStreams = HELIX_A2A_STATIC_MAX_STREAMS;
+constexpr size_t kStaticScratchBytes = static_cast<size_t>(kStaticStreams) * (kFifoBytes + 2 * kFifoInfoBytes);
+static __device__ __align__(256) uint8_t scratch[kStaticScratchBytes];
 
 int device_state(DeviceState** out) {
   int dev = 0;
@@ -86,6 +97,11 @@ int device_state(DeviceState** out) {
     if (st.initError != hipSuccess) return;
     st.status = static_cast<uint32_t*>(p);
     st.initError = hipMemset(st.status, 0, sizeof(uint32_t) * 4);
+    if (st.initError != hipSuccess) return;
+    void* sp = nullptr;
+    st.initError = hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch));
+    if (st.initError != hipSuccess) return;
+    st.scratch = static_cast<uint8_t*>(sp);
   });
   if (st.initError != hipSuccess)
     return fail(HELIX_A2A_ERR_RUNTIME, "device %d setup failed: %s", dev, hipGetErrorString(st.initError));
@@ -406,6 +422,42 @@ int helix_a2a_alltoall_loopback(const helix_a2a_params_t* per_rank, int cp_size,
   int rc = build_plan(per_rank, cp_size, true, &plan);
   if (rc) return rc;
   return launch_rounds(plan, true, true, true, static_cast<hipStream_t>(stream));
+}
+
+int helix_a2a_alltoall_loopback_static(const helix_a2a_params_t* per_rank, int cp_size, int reset, void* stream) {
+  if (per_rank == nullptr) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "no rank descriptors given");
+  int rc = check_cp_size(cp_size);
+  if (rc) return rc;
+  if (per_rank[0].cp_size != cp_size || per_rank[0].cp_rank != 0)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "loopback needs descriptors of ranks 0..cp_size-1 in order");
+  if (cp_size * cp_size > kStaticStreams)
+    return fail(HELIX_A2A_ERR_CAPACITY,
+                "the built-in workspace holds %d FIFOs, cp_size %d needs at least %d (cp_size <= %d); "
+                "use helix_a2a_alltoall_loopback with a workspace of your own",
+                kStaticStreams, cp_size, cp_size * cp_size, HELIX_A2A_STATIC_MAX_CP_SIZE);
+  DeviceState* st = nullptr;
+  if ((rc = device_state(&st))) return rc;
+  BuiltinWorkspace ws;
+  ws.maxChannels = kStaticStreams / (cp_size * cp_size);
+  ws.rowStrideBytes = workspace_bytes(cp_size, ws.maxChannels);
+  ws.base = st->scratch;  // the device address from hipGetSymbolAddress, never the array's name
+  Plan plan;
+  if ((rc = build_plan(per_rank, cp_size, true, &plan, &ws))) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  {
+    // The array keeps the last call's contents. Its layout depends on cp_size, so a change of cp_size
+    // (or the first call, or a caller's request) lays it out again: FIFO bytes 0xFF, counters 0, by a
+    // fill kernel in stream order ahead of the exchange.
+    std::lock_guard<std::mutex> lock(st->scratchMutex);
+    if (reset || st->scratchCp != cp_size) {
+      for (int r = 0; r < cp_size; ++r)
+        HELIX_HIP_TRY(launch_init_row(ws.base + static_cast<uint64_t>(r) * ws.rowStrideBytes,
+                                      fifo_region_bytes(cp_size, ws.maxChannels),
+                                      2 * info_region_bytes(cp_size, ws.maxChannels), s));
+      st->scratchCp = cp_size;
+    }
+  }
+  return launch_rounds(plan, true, true, true, s);
 }
 
 int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, const helix_a2a_combine_out_t* out,

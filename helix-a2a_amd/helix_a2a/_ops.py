@@ -79,6 +79,8 @@ def _load_library() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.argtypes = [P(_Params), ctypes.c_int, ctypes.c_void_p]
         fn.restype = ctypes.c_int
+    lib.helix_a2a_alltoall_loopback_static.argtypes = [P(_Params), ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.helix_a2a_alltoall_loopback_static.restype = ctypes.c_int
     lib.helix_a2a_set_units_per_wavefront.argtypes = [ctypes.c_int]
     lib.helix_a2a_set_units_per_wavefront.restype = ctypes.c_int
     lib.helix_a2a_alltoall_combine_loopback.argtypes = [
@@ -361,6 +363,33 @@ def alltoall_loopback(partial_o: Sequence[torch.Tensor], softmax_stats: Sequence
             arr[r] = _make_params(o3, s3, oo.view(o3.shape), os_.view(s3.shape), workspace, r, cp_size, channel_count)
         _check(_lib.helix_a2a_alltoall_loopback(arr, cp_size, _stream_handle()), "alltoall_loopback")
     return outs_o, outs_s
+
+
+def alltoall_loopback_static(partial_o: Sequence[torch.Tensor], softmax_stats: Sequence[torch.Tensor],
+                             out: Tuple[Sequence[torch.Tensor], Sequence[torch.Tensor]], channel_count: int = 0,
+                             reset: bool = False) -> None:
+    """Loopback exchange into ``out`` through the workspace built into the library (no allocation anywhere).
+
+    At most ``cp_size = 11`` ranks; calls on one GPU must be ordered with respect to each other.
+    """
+    cp_size = len(partial_o)
+    _require(1 <= cp_size <= MAX_CP_SIZE and len(softmax_stats) == cp_size and len(out[0]) == cp_size
+             and len(out[1]) == cp_size, "need one partial_o, softmax_stats and output pair per rank")
+    arr = (_Params * cp_size)()
+    shape0 = None
+    with torch.cuda.device(partial_o[0].device):
+        for r in range(cp_size):
+            o3, s3 = _as_3d(partial_o[r], softmax_stats[r], cp_size)
+            sig = (tuple(o3.shape), tuple(s3.shape), partial_o[r].dtype)
+            shape0 = shape0 or sig
+            _require(sig == shape0, "all ranks must exchange tensors of one shape and dtype")
+            oo, os_ = out[0][r], out[1][r]
+            _require(oo.shape == partial_o[r].shape and oo.dtype == partial_o[r].dtype and oo.is_contiguous()
+                     and os_.shape == softmax_stats[r].shape and os_.dtype == torch.float32 and os_.is_contiguous()
+                     and oo.is_cuda and os_.is_cuda, "out tensors must match the inputs")
+            arr[r] = _make_params(o3, s3, oo.view(o3.shape), os_.view(s3.shape), None, r, cp_size, channel_count)
+        _check(_lib.helix_a2a_alltoall_loopback_static(arr, cp_size, 1 if reset else 0, _stream_handle()),
+               "alltoall_loopback_static")
 
 
 class LoopbackPlan:

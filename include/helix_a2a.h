@@ -37,6 +37,10 @@ extern "C" {
 #define HELIX_A2A_MAX_CP_SIZE 32
 #define HELIX_A2A_MAX_COMBINE_CP_SIZE 32 /* helix_a2a_alltoall_combine_loopback */
 
+/* helix_a2a_alltoall_loopback_static: FIFOs the built-in workspace holds, and the largest cp_size that fits */
+#define HELIX_A2A_STATIC_MAX_STREAMS 128
+#define HELIX_A2A_STATIC_MAX_CP_SIZE 11
+
 /* error codes */
 #define HELIX_A2A_OK 0
 #define HELIX_A2A_ERR_INVALID_ARGUMENT 1 /* a parameter failed validation        */
@@ -174,6 +178,33 @@ int helix_a2a_alltoall_recv(const helix_a2a_params_t* per_rank, int rank_count, 
  *   recv_r[e, s, :] = send_s[e, r, :]     for both fields.
  */
 int helix_a2a_alltoall_loopback(const helix_a2a_params_t* per_rank, int cp_size, void* stream);
+
+/*
+ * helix_a2a_alltoall_loopback without a workspace argument and without any
+ * allocation. No counterpart in the reference; it is for callers that cannot
+ * allocate device memory at this point (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc). The FIFOs live in a
+ * workspace built into the library: a device array of
+ * HELIX_A2A_STATIC_MAX_STREAMS x (512 KiB + 512 B) = 67 174 400 bytes that
+ * every GPU the library runs on holds until the process ends. The workspace
+ * members of the descriptors must be NULL / 0 (max_channel_count is ignored);
+ * everything else is as for helix_a2a_alltoall_loopback, same results.
+ *   limit   cp_size * cp_size <= HELIX_A2A_STATIC_MAX_STREAMS, i.e. cp_size <= 11
+ *           (HELIX_A2A_ERR_CAPACITY beyond); the channel count is at most
+ *           128 / cp_size^2, so large exchanges run slower than with a full workspace.
+ *   state   the array keeps its contents between calls. It is laid out again
+ *           (FIFO bytes 0xFF, counters 0, by a fill kernel on `stream`) on the
+ *           first call on a device, when cp_size differs from the previous
+ *           call's, and when `reset` is non-zero (required after a time-out
+ *           reported by helix_a2a_device_status).
+ *   races   all calls on one GPU share that GPU's array: they must be ordered
+ *           with respect to each other (one stream, or events). Calls that
+ *           overlap on one GPU race.
+ * The very first library call on a device performs the one-time set-up
+ * (device query, symbol addresses); make any library call before starting a
+ * graph capture.
+ */
+int helix_a2a_alltoall_loopback_static(const helix_a2a_params_t* per_rank, int cp_size, int reset, void* stream);
 
 /*
  * Loopback exchange fused with the LSE-weighted combine: the receive half

@@ -1,0 +1,100 @@
+"""The entry point that allocates nothing (helix_a2a_alltoall_loopback_static) against
+helix_a2a_alltoall_loopback, through the C ABI: bit-exact, on calls in a row that share the
+built-in workspace (the second smaller than the first, then another cp_size, then a reset)."""
+import ctypes
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hx():
+    import helix_a2a
+
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return helix_a2a
+
+
+@pytest.fixture(scope="module")
+def ops(hx):
+    from helix_a2a import _ops
+
+    return _ops
+
+
+def _inputs(cp, entries, x, s, seed):
+    g = torch.Generator(device="cpu")
+    g.manual_seed(seed)
+    ins_o = [torch.randint(-32768, 32767, (entries, cp, x), generator=g, dtype=torch.int16).view(torch.bfloat16).cuda()
+             for _ in range(cp)]
+    ins_s = [torch.randint(-2**31, 2**31 - 1, (entries, cp, s), generator=g, dtype=torch.int32).view(torch.float32).cuda()
+             for _ in range(cp)]
+    return ins_o, ins_s
+
+
+def _bits_equal(a, b):
+    view = {2: torch.int16, 4: torch.int32}[a.element_size()]
+    return torch.equal(a.view(view), b.view(view))
+
+
+def _both(hx, ops, ws, cp, entries, x, s, seed, reset=False):
+    ins_o, ins_s = _inputs(cp, entries, x, s, seed)
+    want_o, want_s = hx.alltoall_loopback(ins_o, ins_s, ws)
+    got_o = [torch.full_like(t, 7.0) for t in ins_o]
+    got_s = [torch.full_like(t, 7.0) for t in ins_s]
+    torch.cuda.synchronize()
+    ops.alltoall_loopback_static(ins_o, ins_s, (got_o, got_s), reset=reset)
+    torch.cuda.synchronize()
+    assert ops.device_status() == 0
+    for r in range(cp):
+        assert _bits_equal(got_o[r], want_o[r]), f"partial_o of rank {r} differs (cp={cp}, entries={entries})"
+        assert _bits_equal(got_s[r], want_s[r]), f"softmax_stats of rank {r} differs (cp={cp}, entries={entries})"
+
+
+def test_static_loopback_matches_the_workspace_entry_point(hx, ops):
+    cp = 4
+    ws = hx.allocate_workspace(cp, 0)
+    for r in range(cp):
+        hx.init_workspace(ws, r, cp)
+    _both(hx, ops, ws, cp, 64, 32 * 128, 64, seed=1)      # c2's shape
+    _both(hx, ops, ws, cp, 37, 6 * 96, 12, seed=2)        # smaller, ragged: the array still holds the first call's lines
+    _both(hx, ops, ws, cp, 3, 64, 2, seed=3)              # a few tiny messages
+    for i in range(6):                                    # the FIFO entries wrap (four per stream)
+        _both(hx, ops, ws, cp, 5 + i, 256, 4, seed=10 + i)
+    _both(hx, ops, ws, cp, 2000, 512, 4, seed=4)          # 8 channels x 4 entries cannot hold it: rounds
+    del ws
+    # another cp_size lays the array out again
+    cp = 8
+    ws = hx.allocate_workspace(cp, 0)
+    for r in range(cp):
+        hx.init_workspace(ws, r, cp)
+    _both(hx, ops, ws, cp, 256, 8 * 128, 16, seed=5)      # c3's shape on 2 channels
+    _both(hx, ops, ws, cp, 9, 128, 2, seed=6)
+    _both(hx, ops, ws, cp, 9, 128, 2, seed=7, reset=True)
+    del ws
+    cp = 2
+    ws = hx.allocate_workspace(cp, 0)
+    for r in range(cp):
+        hx.init_workspace(ws, r, cp)
+    _both(hx, ops, ws, cp, 8, 4 * 128, 8, seed=8)
+
+
+def test_static_loopback_limits(hx, ops):
+    cp = 12  # 144 FIFOs: more than the built-in workspace holds
+    ins_o, ins_s = _inputs(cp, 2, 64, 2, seed=9)
+    out = ([torch.empty_like(t) for t in ins_o], [torch.empty_like(t) for t in ins_s])
+    with pytest.raises(RuntimeError, match="built-in workspace holds 128 FIFOs"):
+        ops.alltoall_loopback_static(ins_o, ins_s, out)
+    # a workspace pointer is refused: the call would silently ignore it otherwise
+    cp = 2
+    ins_o, ins_s = _inputs(cp, 2, 64, 2, seed=10)
+    out = ([torch.empty_like(t) for t in ins_o], [torch.empty_like(t) for t in ins_s])
+    arr = (ops._Params * cp)()
+    for r in range(cp):
+        arr[r] = ops._make_params(ins_o[r], ins_s[r], out[0][r], out[1][r], None, r, cp, 0)
+        arr[r].workspace = ins_o[0].data_ptr()
+    assert ops._lib.helix_a2a_alltoall_loopback_static(arr, cp, 0, ops._stream_handle()) == 1
+    assert b"built-in workspace" in ops._lib.helix_a2a_last_error()
+    assert isinstance(ctypes.CDLL(ops.library_path()).helix_a2a_alltoall_loopback_static, ctypes._CFuncPtr)
