@@ -40,6 +40,17 @@ int fail(int code, const char* fmt, ...) {
 
 std::atomic<uint64_t> g_spinLimitUs{2000000};
 std::atomic<int> g_singleRound{0};
+std::atomic<int> g_checked{-1};  // -1: not decided yet (HELIX_A2A_CHECKED is read once)
+
+bool checked_mode() {
+  int v = g_checked.load();
+  if (v < 0) {
+    const char* env = std::getenv("HELIX_A2A_CHECKED");
+    v = (env && *env && std::strcmp(env, "0") != 0) ? 1 : 0;
+    g_checked.store(v);
+  }
+  return v != 0;
+}
 // Units per lane a wavefront takes of a run before the run is shared with another wavefront:
 // -1 = kMaxUnitsInFlight, and only while the launch leaves wavefront slots of the device free;
 // 0 = never share; 1..6 = always share beyond that many.
@@ -349,6 +360,31 @@ int launch_rounds(Plan& plan, bool send, bool recv, bool allowRounds, hipStream_
   return HELIX_A2A_OK;
 }
 
+// Wait for `stream`, read the device status word and clear it.
+int read_status(DeviceState* st, hipStream_t stream, uint32_t* out) {
+  HELIX_HIP_TRY(hipStreamSynchronize(stream));
+  uint32_t host = 0;
+  HELIX_HIP_TRY(hipMemcpy(&host, st->status, sizeof(host), hipMemcpyDeviceToHost));
+  if (host != 0) HELIX_HIP_TRY(hipMemset(st->status, 0, sizeof(uint32_t)));
+  *out = host;
+  return HELIX_A2A_OK;
+}
+
+// End of every exchange call: nothing in the normal mode, a synchronous status check in checked mode.
+int finish_call(int rc, hipStream_t stream) {
+  if (rc != HELIX_A2A_OK || !checked_mode()) return rc;
+  DeviceState* st = nullptr;
+  if ((rc = device_state(&st))) return rc;
+  uint32_t status = 0;
+  if ((rc = read_status(st, stream, &status))) return rc;
+  if (status == 0) return HELIX_A2A_OK;
+  return fail(HELIX_A2A_ERR_DEVICE, "the exchange raised device status 0x%x (%s%s%s%s); re-initialise the workspace", status,
+              (status & HELIX_A2A_STATUS_RECV_TIMEOUT) ? "receive wait timed out " : "",
+              (status & HELIX_A2A_STATUS_SEND_TIMEOUT) ? "send wait timed out " : "",
+              (status & HELIX_A2A_STATUS_INTERNAL) ? "corrupt line " : "",
+              (status & HELIX_A2A_STATUS_BROKEN_WORKSPACE) ? "workspace broken by an earlier failure" : "");
+}
+
 }  // namespace
 
 extern "C" {
@@ -397,7 +433,8 @@ int helix_a2a_alltoall(const helix_a2a_params_t* params, void* stream) {
   if (rc) return rc;
   // both halves in one launch: with peers on the same queue behind this call
   // the receive half can only time out, so rounds are not an option here
-  return launch_rounds(plan, true, true, plan.args.cpSize == 1, static_cast<hipStream_t>(stream));
+  return finish_call(launch_rounds(plan, true, true, plan.args.cpSize == 1, static_cast<hipStream_t>(stream)),
+                     static_cast<hipStream_t>(stream));
 }
 
 int helix_a2a_alltoall_send(const helix_a2a_params_t* per_rank, int rank_count, void* stream) {
@@ -411,7 +448,8 @@ int helix_a2a_alltoall_recv(const helix_a2a_params_t* per_rank, int rank_count, 
   Plan plan;
   int rc = build_plan(per_rank, rank_count, true, &plan);
   if (rc) return rc;
-  return launch_rounds(plan, false, true, false, static_cast<hipStream_t>(stream));
+  return finish_call(launch_rounds(plan, false, true, false, static_cast<hipStream_t>(stream)),
+                     static_cast<hipStream_t>(stream));
 }
 
 int helix_a2a_alltoall_loopback(const helix_a2a_params_t* per_rank, int cp_size, void* stream) {
@@ -421,7 +459,7 @@ int helix_a2a_alltoall_loopback(const helix_a2a_params_t* per_rank, int cp_size,
   Plan plan;
   int rc = build_plan(per_rank, cp_size, true, &plan);
   if (rc) return rc;
-  return launch_rounds(plan, true, true, true, static_cast<hipStream_t>(stream));
+  return finish_call(launch_rounds(plan, true, true, true, static_cast<hipStream_t>(stream)), static_cast<hipStream_t>(stream));
 }
 
 int helix_a2a_alltoall_loopback_static(const helix_a2a_params_t* per_rank, int cp_size, int reset, void* stream) {
@@ -457,7 +495,7 @@ int helix_a2a_alltoall_loopback_static(const helix_a2a_params_t* per_rank, int c
       st->scratchCp = cp_size;
     }
   }
-  return launch_rounds(plan, true, true, true, s);
+  return finish_call(launch_rounds(plan, true, true, true, s), s);
 }
 
 int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, const helix_a2a_combine_out_t* out,
@@ -521,7 +559,7 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, cons
     a.doRecv = 1;
     HELIX_HIP_TRY(launch_combine(a, static_cast<int>(parts), static_cast<hipStream_t>(stream)));
   }
-  return HELIX_A2A_OK;
+  return finish_call(HELIX_A2A_OK, static_cast<hipStream_t>(stream));
 }
 
 int helix_a2a_device_status(uint32_t* status, void* stream) {
@@ -529,14 +567,10 @@ int helix_a2a_device_status(uint32_t* status, void* stream) {
   DeviceState* st = nullptr;
   int rc = device_state(&st);
   if (rc) return rc;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  HELIX_HIP_TRY(hipStreamSynchronize(s));
-  uint32_t host = 0;
-  HELIX_HIP_TRY(hipMemcpy(&host, st->status, sizeof(host), hipMemcpyDeviceToHost));
-  if (host != 0) HELIX_HIP_TRY(hipMemset(st->status, 0, sizeof(uint32_t)));
-  *status = host;
-  return HELIX_A2A_OK;
+  return read_status(st, static_cast<hipStream_t>(stream), status);
 }
+
+void helix_a2a_set_checked_mode(int enabled) { g_checked.store(enabled ? 1 : 0); }
 
 void helix_a2a_set_spin_limit_us(uint64_t microseconds) { g_spinLimitUs.store(microseconds); }
 

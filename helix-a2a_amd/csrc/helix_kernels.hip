@@ -68,6 +68,7 @@ constexpr int kDppWaveShl1 = 0x130;  // DPP control: lane i reads lane i + 1 of 
 constexpr uint32_t kStatusRecvTimeout = 1u;
 constexpr uint32_t kStatusSendTimeout = 2u;
 constexpr uint32_t kStatusInternal = 4u;
+constexpr uint32_t kStatusBrokenWorkspace = 8u;
 
 // Units a lane keeps in flight per pass over a run: at most kMaxUnitsInFlight
 // (6 x 16 B x 64 lanes = 6 KiB per wavefront), and no more than the runs of a
@@ -108,12 +109,16 @@ __device__ uint64_t g_timeline[kTimelineWaves * 4];
   } while (0)
 #endif
 
-// Bounded wait bookkeeping. The clock is read every 64th spin only.
+// Bounded wait bookkeeping. Every 64th spin reads the clock and the workspace's broken word: a wait
+// ends when its time is up or when another wavefront has given up on this workspace already, so that
+// a failed launch drains at once instead of one time limit after the other.
 struct SpinGuard {
   uint64_t limit;
   uint64_t start;
+  const uint64_t* broken;
   uint32_t spins;
-  __device__ __forceinline__ explicit SpinGuard(uint64_t limitTicks) : limit(limitTicks), start(0), spins(0) {}
+  __device__ __forceinline__ SpinGuard(uint64_t limitTicks, const uint64_t* brokenWord)
+      : limit(limitTicks), start(0), broken(brokenWord), spins(0) {}
   __device__ __forceinline__ bool expired() {
     spins += 1;
     if ((spins & 63u) != 1u) return false;
@@ -122,6 +127,7 @@ struct SpinGuard {
       start = now;
       return limit == 0;
     }
+    if (__hip_atomic_load(broken, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return true;
     return now - start > limit;
   }
 };
@@ -136,8 +142,29 @@ __device__ __forceinline__ uint32_t lane_value(uint32_t v, int q) {
   return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), q));
 }
 
-__device__ __forceinline__ void raise_status(uint32_t* status, uint32_t bits, int lane) {
-  if (lane == 0) atomicOr(status, bits);
+__device__ __forceinline__ uint64_t* broken_word(const KernelArgs& a) {
+  return reinterpret_cast<uint64_t*>(a.workspace + broken_word_offset(a.cpSize, a.maxChannels));
+}
+
+// Whether the workspace was broken before this launch started. A wave-uniform read through the scalar
+// cache (which starts every launch empty): it costs no vector memory instruction, and it need not see
+// what the running launch does to the word -- the bounded waits look at that themselves.
+__device__ __forceinline__ uint64_t broken_at_launch(const KernelArgs& a) {
+  using ConstWord = const __attribute__((address_space(4))) uint64_t;
+  return *reinterpret_cast<ConstWord*>(reinterpret_cast<uintptr_t>(broken_word(a)));
+}
+
+// A failure: the status word of the device tells the host, the broken word of the workspace tells every
+// wavefront that comes later (of this launch and of the launches behind it).
+__device__ __forceinline__ void raise_status(const KernelArgs& a, uint32_t bits, int lane) {
+  if (lane == 0) {
+    atomicOr(a.status, bits);
+    __hip_atomic_fetch_or(broken_word(a), static_cast<uint64_t>(bits), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+// The workspace was broken before this wavefront started: it reports that and does nothing.
+__device__ __forceinline__ void report_broken(const KernelArgs& a, int lane) {
+  if (lane == 0) atomicOr(a.status, kStatusBrokenWorkspace);
 }
 
 // What a stream's wavefront needs to know, all wave-uniform.
@@ -221,6 +248,7 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
   // the counters are only needed once the first payload loads are in flight
   int64_t step = *token;
   int64_t tail = info[1];
+  const uint64_t broken = broken_at_launch(a);
 
   for (int firstMsg = 0; firstMsg < st.msgs; firstMsg += st.msgsPerEntry) {
     const int runMsgs = min(st.msgsPerEntry, st.msgs - firstMsg);
@@ -230,17 +258,21 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
     // open the FIFO entry of this run (csrc/helix_alltoall.cu:377-390); false when the wait for room gave up
     auto open_entry = [&]() -> bool {
       opened = true;
+      if (broken != 0) {
+        report_broken(a, lane);
+        return false;
+      }
       if (firstMsg > 0) {
         step += 1;
         wait_stores_acknowledged();
         if (lane == 0) st_counter(token, step);
       }
-      SpinGuard guard(a.spinLimitTicks);
+      SpinGuard guard(a.spinLimitTicks, broken_word(a));
       while (tail + kFifoDepth <= step) {  // the entry is free once the receiver released step - 4
         tail = ld_counter(&info[1]);
         if (tail + kFifoDepth > step) break;
         if (guard.expired()) {
-          raise_status(a.status, kStatusSendTimeout, lane);
+          raise_status(a, kStatusSendTimeout, lane);
           return false;
         }
         __builtin_amdgcn_s_sleep(4);
@@ -328,6 +360,10 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
 
   int64_t step = *mine;
   int64_t head = ld_counter(token);
+  if (broken_at_launch(a) != 0) {
+    report_broken(a, lane);
+    return;
+  }
 
   for (int firstMsg = 0; firstMsg < st.msgs; firstMsg += st.msgsPerEntry) {
     const int runMsgs = min(st.msgsPerEntry, st.msgs - firstMsg);
@@ -343,12 +379,12 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
       }
     }
     if (head <= step) {
-      SpinGuard guard(a.spinLimitTicks);
+      SpinGuard guard(a.spinLimitTicks, broken_word(a));
       for (;;) {
         head = ld_counter(token);
         if (head > step) break;
         if (guard.expired()) {
-          raise_status(a.status, kStatusRecvTimeout, lane);
+          raise_status(a, kStatusRecvTimeout, lane);
           return;
         }
         __builtin_amdgcn_s_sleep(1);
@@ -375,7 +411,7 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
         flagsAgree &= U >= passEnd || (U & 7u) != 7u || (v[i].z == stepLo && v[i].w == stepHi);
       }
       if (__ballot(!flagsAgree) != 0ull) {
-        raise_status(a.status, kStatusInternal, lane);
+        raise_status(a, kStatusInternal, lane);
         return;
       }
       if (U0 == slice.begin && firstMsg == 0) HELIX_MARK(wave, 1, false);
@@ -618,7 +654,12 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
     mySenderInfo = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(a.cpSize, a.maxChannels, r, ch));
     myStep = myInfo[1];
   }
+  const bool broken = broken_at_launch(a) != 0;
   __syncthreads();  // every part has read the counters before part 0 moves them
+  if (broken) {
+    report_broken(a, lane);
+    return;
+  }
   if (part == 0 && lane < a.cpSize) {
     // rounds never put more than the four entries in flight, so the entries can
     // be handed back up front; nothing reads these counters before the launch ends
@@ -637,12 +678,12 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
       // Acquire the run from every sender: a head beyond the step says that all
       // lines of the step are in memory (the sender waits for its stores before
       // it moves head). Every unit needs all cpSize senders anyway.
-      SpinGuard guard(a.spinLimitTicks);
+      SpinGuard guard(a.spinLimitTicks, broken_word(a));
       for (;;) {
         const bool closed = lane >= a.cpSize || ld_counter(&mySenderInfo[0]) > myStep;
         if (__ballot(!closed) == 0ull) break;
         if (guard.expired()) {
-          raise_status(a.status, kStatusRecvTimeout, lane);
+          raise_status(a, kStatusRecvTimeout, lane);
           return;
         }
         __builtin_amdgcn_s_sleep(8);
@@ -696,7 +737,7 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
       const int slotB = ownB ? slotA + 1 : slotA;
       const int slotCount = __popcll(startsA) + __popcll(startsB);
       if (slotCount > kCombineSlots) {  // excluded by the host's shape check (head_dim >= 32)
-        raise_status(a.status, kStatusInternal, lane);
+        raise_status(a, kStatusInternal, lane);
         return;
       }
       if (newA) {
@@ -780,7 +821,7 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
       }
       if (__ballot(flagMismatch != 0u) != 0ull) {
         // the head tokens promised complete lines: a flag that disagrees means the workspace is corrupt
-        raise_status(a.status, kStatusInternal, lane);
+        raise_status(a, kStatusInternal, lane);
         return;
       }
       __builtin_amdgcn_raw_buffer_store_b64(narrow_piece<kDtype>(accA), outRsrc,

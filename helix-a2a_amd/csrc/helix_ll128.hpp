@@ -213,6 +213,11 @@ HELIX_HD int units_in_flight_for_run(long runUnits) {
 // launches may differ in their number of parts.
 constexpr int kCounterSlots = kFifoInfoBytes / 8;     // 32
 constexpr int kMaxStreamParts = 16;
+// The last slot of the very first sender counter block of row 0 (receiver 0, channel 0) is the workspace's
+// "broken" word: a kernel whose wait gave up, or that met a corrupt line, leaves its status bits there,
+// and every later wavefront that finds it non-zero does nothing. Initialising row 0 clears it.
+constexpr int kBrokenSlot = kCounterSlots - 1;
+HELIX_HD uint64_t broken_word_offset(int cpSize, int maxCh) { return sender_info_offset(cpSize, maxCh, 0, 0) + kBrokenSlot * 8ull; }
 HELIX_HD int sender_counter_slot(int part) { return part == 0 ? 0 : part + 1; }
 HELIX_HD int receiver_counter_slot(int part) { return part + 1; }
 

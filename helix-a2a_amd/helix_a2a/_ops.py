@@ -90,6 +90,8 @@ def _load_library() -> ctypes.CDLL:
     lib.helix_a2a_device_status.restype = ctypes.c_int
     lib.helix_a2a_set_spin_limit_us.argtypes = [ctypes.c_uint64]
     lib.helix_a2a_set_spin_limit_us.restype = None
+    lib.helix_a2a_set_checked_mode.argtypes = [ctypes.c_int]
+    lib.helix_a2a_set_checked_mode.restype = None
     lib.helix_a2a_set_single_round.argtypes = [ctypes.c_int]
     lib.helix_a2a_set_single_round.restype = None
     lib.helix_a2a_last_error.argtypes = []
@@ -606,6 +608,17 @@ def set_spin_limit_us(microseconds: int) -> None:
 def set_units_per_wavefront(units: int) -> None:
     """Share a stream's runs longer than ``units`` KiB between wavefronts: 1..6 always, 0 never, -1 (default) beyond 6 KiB while the launch leaves the device under-filled."""
     _check(_lib.helix_a2a_set_units_per_wavefront(int(units)), "set_units_per_wavefront")
+
+
+def set_checked_mode(enabled: bool) -> None:
+    """Every exchange call waits for its stream and raises if a kernel reported a failure (bring-up, tests)."""
+    _lib.helix_a2a_set_checked_mode(1 if enabled else 0)
+
+
+STATUS_RECV_TIMEOUT = 1
+STATUS_SEND_TIMEOUT = 2
+STATUS_INTERNAL = 4
+STATUS_BROKEN_WORKSPACE = 8
 
 
 def set_single_round(enabled: bool) -> None:

@@ -46,11 +46,13 @@ extern "C" {
 #define HELIX_A2A_ERR_INVALID_ARGUMENT 1 /* a parameter failed validation        */
 #define HELIX_A2A_ERR_RUNTIME 2          /* a HIP runtime call failed            */
 #define HELIX_A2A_ERR_CAPACITY 3         /* traffic does not fit the FIFOs in the requested mode */
+#define HELIX_A2A_ERR_DEVICE 4           /* checked mode: the exchange raised bits in the device status word */
 
 /* bits of the device status word (helix_a2a_device_status) */
 #define HELIX_A2A_STATUS_RECV_TIMEOUT 1u /* a receiver gave up polling for a line */
 #define HELIX_A2A_STATUS_SEND_TIMEOUT 2u /* a sender gave up waiting for FIFO room */
 #define HELIX_A2A_STATUS_INTERNAL 4u     /* a kernel met a state its launch checks exclude (corrupt workspace) */
+#define HELIX_A2A_STATUS_BROKEN_WORKSPACE 8u /* an exchange did nothing: an earlier failure left its workspace unusable */
 
 /*
  * One field of a message. Same members and meaning as the reference's
@@ -223,6 +225,28 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank,
  * No counterpart in the reference, whose waits are unbounded.
  */
 int helix_a2a_device_status(uint32_t* status, void* stream);
+
+/*
+ * What a failure inside a kernel does. The reference's waits are unbounded: a
+ * peer that never sends hangs the GPU. Here a wait that exceeds the spin limit,
+ * or a line whose flag disagrees with its token, ends the wavefront, raises its
+ * bit in the device status word and marks the workspace broken (a word in row
+ * 0's counter region). Every wavefront that runs afterwards on that workspace
+ * -- the rest of the launch and every launch queued behind it -- writes nothing
+ * and raises HELIX_A2A_STATUS_BROKEN_WORKSPACE, so the output tensors of
+ * such an exchange keep whatever they held before; the FIFO counters are no
+ * longer consistent. helix_a2a_init_workspace on row 0 (with the other rows)
+ * makes the workspace usable again. The calls themselves return at launch, so
+ * a caller learns of a failure from helix_a2a_device_status, or at once in
+ * checked mode:
+ *
+ * helix_a2a_set_checked_mode(1): every exchange call waits for its stream and
+ * reads the status word before it returns, and returns HELIX_A2A_ERR_DEVICE
+ * (message: the bits) if it is not zero. For bring-up and tests; it makes the
+ * calls synchronous. Default 0. The environment variable HELIX_A2A_CHECKED=1
+ * switches it on from the start.
+ */
+void helix_a2a_set_checked_mode(int enabled);
 
 /*
  * Upper bound, in microseconds, of any single in-kernel wait (receiver line

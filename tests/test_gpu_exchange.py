@@ -567,6 +567,63 @@ def test_receive_without_send_times_out_cleanly(hx, ops):
         hx.init_workspace(ws, r, cp)
 
 
+def test_exchange_after_a_timeout_does_nothing_until_reinit(hx, ops):
+    # a wait that gives up marks the workspace broken: the exchanges queued behind it write nothing and say so
+    cp = 4
+    ws = get_workspace(hx, cp, fresh=True)
+    g = torch.Generator().manual_seed(77)
+    o = [torch.randint(-32768, 32767, (24, cp, 256), generator=g, dtype=torch.int16).view(torch.bfloat16).cuda() for _ in range(cp)]
+    s = [torch.randint(-2**31, 2**31 - 1, (24, cp, 4), generator=g, dtype=torch.int32).view(torch.float32).cuda() for _ in range(cp)]
+    out_o = [torch.empty_like(t) for t in o]
+    out_s = [torch.empty_like(t) for t in s]
+    arr = (ops._Params * cp)()
+    for r in range(cp):
+        arr[r] = ops._make_params(o[r], s[r], out_o[r], out_s[r], ws, r, cp, 0)
+    ops.set_spin_limit_us(0)  # the receivers' wait gives up at its first clock check; every kernel still exits normally
+    try:
+        ops._check(ops._lib.helix_a2a_alltoall_recv(arr, cp, ops._stream_handle()), "recv")
+        torch.cuda.synchronize()
+    finally:
+        ops.set_spin_limit_us(2_000_000)
+    assert ops.device_status() & ops.STATUS_RECV_TIMEOUT
+    # a complete exchange on the same workspace, with normal limits, without re-initialising
+    sentinel_o = [torch.full_like(t, 3.0) for t in o]
+    sentinel_s = [torch.full_like(t, 3.0) for t in s]
+    hx.alltoall_loopback(o, s, ws, out=(sentinel_o, sentinel_s))
+    comb = torch.full((24, 256), 5.0, dtype=torch.bfloat16, device="cuda")
+    plan = ops.CombinePlan(o, s, ws, ops.STATS_LSE, False, 0)
+    for c in plan.combined:
+        c.fill_(5.0)
+    plan.run()
+    torch.cuda.synchronize()
+    status = ops.device_status()
+    assert status == ops.STATUS_BROKEN_WORKSPACE, f"status {status:#x}"
+    for r in range(cp):
+        assert (sentinel_o[r] == 3.0).all() and (sentinel_s[r] == 3.0).all(), "a broken workspace must not produce output"
+        assert torch.equal(plan.combined[r], comb)
+    # checked mode turns the same condition into an error of the call
+    ops.set_checked_mode(True)
+    try:
+        with pytest.raises(RuntimeError, match="workspace broken by an earlier failure"):
+            hx.alltoall_loopback(o, s, ws)
+    finally:
+        ops.set_checked_mode(False)
+    assert ops.device_status() == 0  # the checked call has read and cleared it
+    for r in range(cp):
+        hx.init_workspace(ws, r, cp)
+    outs_o, outs_s = hx.alltoall_loopback(o, s, ws)
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(o, s, outs_o, outs_s)
+    # and checked mode is silent on a healthy exchange
+    ops.set_checked_mode(True)
+    try:
+        outs_o, outs_s = hx.alltoall_loopback(o, s, ws)
+        check_against_oracle(o, s, outs_o, outs_s, with_numpy=False)
+    finally:
+        ops.set_checked_mode(False)
+
+
 def test_send_capacity_is_checked_for_split_phases(hx, ops):
     # 17-piece messages on one channel: 4 x 903 fit the four FIFO entries; a send-only launch of more is refused
     cp, entries = 2, 3613
