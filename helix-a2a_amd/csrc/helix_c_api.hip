@@ -177,18 +177,18 @@ struct Plan {
 };
 
 int check_field(const helix_a2a_field_t& f, const char* name, int eltSize, int entryCount, int cpSize,
-                bool needData) {
+                bool needData, int align = kPieceBytes) {
   if (needData && f.data == nullptr) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%s: data pointer is null", name);
   if (f.element_size != eltSize)
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%s: element size must be %d bytes, got %d", name, eltSize,
                 f.element_size);
   if (f.element_count <= 0) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%s: element count must be positive", name);
   long bytes = static_cast<long>(f.element_count) * f.element_size;
-  if (f.stride_bytes < bytes || (f.stride_bytes % kPieceBytes) != 0)
-    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%s: row stride %d must be a multiple of 8 and >= row size %ld", name,
-                f.stride_bytes, bytes);
-  if ((reinterpret_cast<uintptr_t>(f.data) % kPieceBytes) != 0)
-    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%s: data pointer must be 8-byte aligned", name);
+  if (f.stride_bytes < bytes || (f.stride_bytes % align) != 0)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%s: row stride %d must be a multiple of %d and >= row size %ld", name,
+                f.stride_bytes, align, bytes);
+  if ((reinterpret_cast<uintptr_t>(f.data) % align) != 0)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%s: data pointer must be %d-byte aligned", name, align);
   double extent = static_cast<double>(entryCount) * cpSize * f.stride_bytes;
   if (extent >= 2147483648.0)
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "%s: tensor extent %.0f bytes exceeds 2 GiB", name, extent);
@@ -199,8 +199,9 @@ int check_field(const helix_a2a_field_t& f, const char* name, int eltSize, int e
 // kernel argument block. Checks that need no device come first, so that a
 // malformed descriptor is reported even where no GPU is present. `exchangeOutputs` selects whether recv_fields are
 // checked (exchange) or ignored (combine).
+// `packedStats`: softmax_stats holds one float per head (combine, HELIX_A2A_STATS_LSE_PACKED), any count.
 int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs, Plan* plan,
-               const BuiltinWorkspace* builtin = nullptr) {
+               const BuiltinWorkspace* builtin = nullptr, bool packedStats = false) {
   if (ranks == nullptr || count < 1) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "no rank descriptors given");
   const helix_a2a_params_t& p0 = ranks[0];
   int rc = check_cp_size(p0.cp_size);
@@ -234,7 +235,8 @@ int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs,
       return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "rank descriptors must be consecutive ranks in ascending order");
     const bool haveData = p.entry_count > 0;
     if ((rc = check_field(p.send_fields[0], "send partial_o", 2, p.entry_count, cp, haveData))) return rc;
-    if ((rc = check_field(p.send_fields[1], "send softmax_stats", 4, p.entry_count, cp, haveData))) return rc;
+    if ((rc = check_field(p.send_fields[1], "send softmax_stats", 4, p.entry_count, cp, haveData, packedStats ? 4 : kPieceBytes)))
+      return rc;
     for (int f = 0; f < 2; ++f) {
       if (p.send_fields[f].element_count != p0.send_fields[f].element_count ||
           p.send_fields[f].stride_bytes != p0.send_fields[f].stride_bytes)
@@ -260,7 +262,7 @@ int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs,
   const int f1 = p0.send_fields[1].element_count * 4;
   // csrc/torch_binding.cpp:95-97,105-106
   if (f0 % 16 != 0) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "partial_o rows must be a multiple of 16 bytes, got %d", f0);
-  if (p0.send_fields[1].element_count < 2 || p0.send_fields[1].element_count % 2 != 0)
+  if (!packedStats && (p0.send_fields[1].element_count < 2 || p0.send_fields[1].element_count % 2 != 0))
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "softmax_stats last dimension must be even and >= 2, got %d",
                 p0.send_fields[1].element_count);
   MsgShape sh = make_msg_shape(f0, f1);
@@ -504,16 +506,20 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, cons
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "no rank descriptors or outputs given");
   if (per_rank[0].cp_size != cp_size || per_rank[0].cp_rank != 0)
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "loopback needs descriptors of ranks 0..cp_size-1 in order");
+  const bool base2 = (stats_mode & HELIX_A2A_STATS_BASE2) != 0;
+  stats_mode &= ~HELIX_A2A_STATS_BASE2;
   if (stats_mode != HELIX_A2A_STATS_LSE && stats_mode != HELIX_A2A_STATS_MAX_SUM &&
       stats_mode != HELIX_A2A_STATS_LSE_PACKED)
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "unknown stats_mode %d", stats_mode);
+  if (base2 && stats_mode == HELIX_A2A_STATS_MAX_SUM)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "HELIX_A2A_STATS_BASE2 applies to log-sum-exp statistics, not to (max, sum) pairs");
   if (dtype != HELIX_A2A_DTYPE_BF16 && dtype != HELIX_A2A_DTYPE_FP16)
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "unknown dtype %d", dtype);
   if (cp_size > kMaxCombineCpSize)
     return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "the fused combine serves cp_size <= %d, got %d", kMaxCombineCpSize,
                 cp_size);
   Plan plan;
-  int rc = build_plan(per_rank, cp_size, false, &plan);
+  int rc = build_plan(per_rank, cp_size, false, &plan, nullptr, stats_mode == HELIX_A2A_STATS_LSE_PACKED);
   if (rc) return rc;
   KernelArgs& a = plan.args;
   const int x = per_rank[0].send_fields[0].element_count;
@@ -526,6 +532,7 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, cons
   a.heads = heads;
   a.headDim = x / heads;
   a.statsMode = stats_mode;
+  a.lseBase2 = base2 ? 1 : 0;
   a.dtype = dtype;
   a.headMagic = head_div_magic(static_cast<uint32_t>(a.headDim) * 2u / kPieceBytes);
   const uint64_t outBytes = static_cast<uint64_t>(plan.entryCount) * a.field0Bytes;

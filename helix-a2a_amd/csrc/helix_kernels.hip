@@ -299,9 +299,22 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
         sb[i] = u32x2{0u, 0u};
         if (needField1[i] != 0ull) {
           uint32_t U = U0 + i * kWaveLanes + lane;
-          UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < slice.end);
-          sa[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.a1, 0, kAuxNone);
-          sb[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.b1, 0, kAuxNone);
+          RunUnit d;
+          UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < slice.end, &d);
+          if ((a.field1Bytes & 7) == 0) {
+            sa[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.a1, 0, kAuxNone);
+            sb[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.b1, 0, kAuxNone);
+          } else {
+            // rows of an odd number of floats (one log-sum-exp per head): 4-byte aligned, and the upper
+            // half of a row's last piece is not part of the row -- it travels as zero
+            const uint32_t lastPiece = st.np - 1u;
+            const uint32_t aHi = (o.a1 != kOutOfRange && d.pieceA != lastPiece) ? o.a1 + 4u : kOutOfRange;
+            const uint32_t bHi = (o.b1 != kOutOfRange && d.pieceB != lastPiece) ? o.b1 + 4u : kOutOfRange;
+            sa[i].x = __builtin_amdgcn_raw_buffer_load_b32(st.field1, o.a1, 0, kAuxNone);
+            sa[i].y = __builtin_amdgcn_raw_buffer_load_b32(st.field1, aHi, 0, kAuxNone);
+            sb[i].x = __builtin_amdgcn_raw_buffer_load_b32(st.field1, o.b1, 0, kAuxNone);
+            sb[i].y = __builtin_amdgcn_raw_buffer_load_b32(st.field1, bHi, 0, kAuxNone);
+          }
         }
       }
 #pragma unroll
@@ -614,9 +627,12 @@ __device__ __forceinline__ float fast_log(float x) { return __builtin_amdgcn_log
 // NaN and +-inf count as "no contribution".
 //   mode 0: piece h = {lse, unused}     mode 1: piece h = {running max, running sum}
 //   mode 2: piece h/2 = {lse of head 2*(h/2), lse of head 2*(h/2)+1}
-__device__ __forceinline__ float lse_of_stats(uint32_t s0, uint32_t s1, int statsMode, uint32_t h) {
+// With base2 the log-sum-exp values are base-2 logarithms (the is_lse_base_on_e=False of
+// patches/dcp_alltoall_helix.py:183-186); they are brought to natural logarithms here.
+__device__ __forceinline__ float lse_of_stats(uint32_t s0, uint32_t s1, int statsMode, uint32_t h, bool base2) {
   float x = __uint_as_float((statsMode == 2 && (h & 1u)) ? s1 : s0);
   if (statsMode == 1) x = x + fast_log(__uint_as_float(s1));  // running max + ln(running sum)
+  else if (base2) x *= 0.6931471805599453f;
   return (isnan(x) || isinf(x)) ? -INFINITY : x;
 }
 
@@ -769,7 +785,7 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
         const uint32_t qStepLo = shuffle_from(cx.stepLo, q < a.cpSize ? q : 0);
         const uint32_t off = entry_base(cx, q, qStepLo) + ls * kLineBytes + word * kPieceBytes;
         const u32x2 sv = __builtin_amdgcn_raw_buffer_load_b64(cx.fifos, serving ? off : kOutOfRange, 0, kAuxSc1);
-        const float lse = serving ? lse_of_stats(sv.x, sv.y, a.statsMode, h) : -INFINITY;
+        const float lse = serving ? lse_of_stats(sv.x, sv.y, a.statsMode, h, a.lseBase2 != 0) : -INFINITY;
         float m = lse;
 #pragma unroll
         for (int x = 1; x < kLanesPerSlot; x <<= 1) m = fmaxf(m, shuffle_xor(m, x));
@@ -781,7 +797,8 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
         for (int x = 1; x < kLanesPerSlot; x <<= 1) total += shuffle_xor(total, x);
         if (serving) lds.weight[part][slotSafe][q] = e / fmaxf(total, 1e-10f);
         // one lane per slot reports the head's combined log-sum-exp
-        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(fast_log(total) + m), lseRsrc,
+        const float combinedLse = fast_log(total) + m;
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(a.lseBase2 ? combinedLse * 1.4426950408889634f : combinedLse), lseRsrc,
                                               (serving && q == 0) ? (slotEntry * a.heads + h) * 4u : kOutOfRange, 0,
                                               kAuxNone);
       }

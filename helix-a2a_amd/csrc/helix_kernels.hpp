@@ -27,7 +27,7 @@ struct KernelArgs {
   int maxChannels;          // layout constant of the workspace
   int runChannels;          // channels this launch deals entries over
   int entryBegin, entryEnd; // entries [entryBegin, entryEnd) of the call
-  int field0Bytes, field1Bytes;
+  int field0Bytes, field1Bytes;  // field1Bytes is a multiple of 8, or of 4 for the packed per-head statistics of the combine
   int sendStride0, sendStride1;  // bytes between consecutive (entry, peer) rows
   int recvStride0, recvStride1;
   uint32_t sendBytes0, sendBytes1;  // extent of each tensor (< 2 GiB), the range of its buffer descriptor
@@ -43,6 +43,7 @@ struct KernelArgs {
   // combine only
   int heads, headDim;
   int statsMode, dtype;
+  int lseBase2;        // the statistics are base-2 logarithms, and so is the combined log-sum-exp that is stored
   uint32_t headMagic;  // head_div_magic(pieces per head)
 };
 

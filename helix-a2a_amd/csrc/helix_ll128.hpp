@@ -112,7 +112,7 @@ struct MsgShape {
 HELIX_HD MsgShape make_msg_shape(int field0Bytes, int field1Bytes) {
   MsgShape s;
   s.np0 = field0Bytes / kPieceBytes;
-  s.np = s.np0 + field1Bytes / kPieceBytes;
+  s.np = s.np0 + (field1Bytes + kPieceBytes - 1) / kPieceBytes;  // a row of an odd number of floats: the last piece is half empty
   s.lines = (s.np + kPiecesPerLine - 1) / kPiecesPerLine;
   return s;
 }

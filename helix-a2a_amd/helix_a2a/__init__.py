@@ -149,17 +149,14 @@ def dcp_a2a_lse_reduce(
     gets back ``[B, H/N, D]``, the exact LSE-weighted combination for its heads
     ``r*H/N .. (r+1)*H/N - 1``, and with ``return_lse`` the combined LSE ``[B, H/N]``.
 
+    Any ``H/N`` is taken (the reference pads each LSE to a pair for its kernel,
+    patches/dcp_alltoall_helix.py:560-567; here the LSE rows travel as they are).
+    ``is_lse_base_on_e=False`` says the LSE values are base-2 logarithms; the
+    combine takes them, and returns the combined LSE, in that base.
+
     No permute is needed on either side: ``[B, H, D]`` *is* ``[B, N, (H/N)*D]``,
     which the exchange takes as it is, and the fused combine writes ``[B, H/N, D]``
     directly (the reference path permutes before and after its kernel,
     patches/dcp_alltoall_helix.py:545-593).
     """
-    if not is_lse_base_on_e:
-        cp_attn_lse = [lse * 0.6931471805599453 for lse in cp_attn_lse]  # base-2 LSE -> natural log
-    res = _ops.dcp_reduce(cp_attn_out, cp_attn_lse, workspace, return_lse, channel_count)
-    if return_lse:
-        combined, lses = res
-        if not is_lse_base_on_e:
-            lses = [t * 1.4426950408889634 for t in lses]
-        return combined, lses
-    return res
+    return _ops.dcp_reduce(cp_attn_out, cp_attn_lse, workspace, return_lse, channel_count, lse_base2=not is_lse_base_on_e)

@@ -14,6 +14,8 @@ from __future__ import annotations
 import ctypes
 import os
 import threading
+import time
+import weakref
 from pathlib import Path
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -25,6 +27,7 @@ MAX_COMBINE_CP_SIZE = 32
 STATS_LSE = 0          # stats pairs: (natural-log LSE, unused)
 STATS_MAX_SUM = 1      # stats pairs: (running max, running sum)
 STATS_LSE_PACKED = 2   # one natural-log LSE per head, no padding
+STATS_BASE2 = 16       # or-ed to an LSE mode: the LSE values (in and out) are base-2 logarithms
 
 _LIB_NAME = "libhelix_a2a.so"
 
@@ -160,6 +163,25 @@ def auto_channel_count(cp_size: int, entry_count: int, cu_count: int = 0) -> int
 # workspace
 # --------------------------------------------------------------------------
 
+class _on_device:
+    """``torch.cuda.device(d)`` that costs nothing when ``d`` is the current device already (the usual case)."""
+
+    __slots__ = ("ctx",)
+
+    def __init__(self, device: torch.device) -> None:
+        index = device.index
+        self.ctx = None if index is None or index == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            return self.ctx.__exit__(*exc)
+        return False
+
+
 def _check_workspace(workspace: torch.Tensor, cp_size: int) -> None:
     _require(isinstance(workspace, torch.Tensor) and workspace.is_cuda, "workspace must be on the GPU")
     _require(workspace.dtype == torch.int64, "workspace must be int64 (used as uint64)")
@@ -177,7 +199,8 @@ def initialize_workspace(workspace: torch.Tensor, cp_rank: int, cp_size: int) ->
     _require(workspace.size(1) * 8 >= need, f"workspace rows hold {workspace.size(1) * 8} bytes, {need} needed")
     row_ptr = workspace.data_ptr() + cp_rank * workspace.stride(0) * 8
     # a reset starts a new epoch: half-finished exchanges of logical ranks on this workspace are void
-    _groups.pop((workspace.device.index or 0, workspace.data_ptr(), cp_size), None)
+    with _call_lock:
+        _groups.pop((workspace.device.index or 0, workspace.data_ptr(), cp_size), None)
     _reduce_descriptors.clear()
     with torch.cuda.device(workspace.device):
         _check(_lib.helix_a2a_init_workspace(row_ptr, cp_size, 0, _stream_handle()), "init_workspace")
@@ -231,8 +254,20 @@ def _fill_field(field: _Field, t: torch.Tensor) -> None:
     field.stride_bytes = t.stride(1) * t.element_size()
 
 
+_max_channels_cache: Dict[Tuple[int, int], int] = {}
+
+
+def _device_max_channels(cp_size: int) -> int:
+    """max_channel_count of the current device, asked once per (cp_size, device)."""
+    key = (cp_size, torch.cuda.current_device())
+    n = _max_channels_cache.get(key)
+    if n is None:
+        n = _max_channels_cache[key] = max_channel_count(cp_size)
+    return n
+
+
 def _make_params(o3: torch.Tensor, s3: torch.Tensor, out_o: Optional[torch.Tensor], out_s: Optional[torch.Tensor],
-                 workspace: torch.Tensor, cp_rank: int, cp_size: int, channel_count: int) -> _Params:
+                 workspace: Optional[torch.Tensor], cp_rank: int, cp_size: int, channel_count: int) -> _Params:
     p = _Params()
     _fill_field(p.send_fields[0], o3)
     _fill_field(p.send_fields[1], s3)
@@ -247,8 +282,93 @@ def _make_params(o3: torch.Tensor, s3: torch.Tensor, out_o: Optional[torch.Tenso
     if workspace is not None:
         p.workspace = workspace.data_ptr()
         p.workspace_stride_u64 = workspace.stride(0)
-        p.max_channel_count = max_channel_count(cp_size)
+        p.max_channel_count = _device_max_channels(cp_size)
     return p
+
+
+class _ExchangeShape:
+    """What the checks of one (partial_o shape, stats shape, dtype, cp_size) came to, kept so that a serving
+    loop pays for them once: entry count, row widths, and descriptor arrays per workspace that a call only
+    has to put its data pointers into."""
+
+    def __init__(self, partial_o: torch.Tensor, softmax_stats: torch.Tensor, cp_size: int) -> None:
+        o3, s3 = _as_3d(partial_o, softmax_stats, cp_size)  # raises on anything the reference's binding rejects
+        self.cp_size = cp_size
+        self.entries = o3.size(0)
+        self.row0 = o3.size(2)
+        self.row1 = s3.size(2)
+        self.elt = partial_o.element_size()
+        self.shape_o = partial_o.shape
+        self.shape_s = softmax_stats.shape
+        self.dtype = partial_o.dtype
+        self.arrays: Dict[tuple, ctypes.Array] = {}
+
+    def array(self, workspace: torch.Tensor, channel_count: int) -> ctypes.Array:
+        """The cp descriptors of this shape on this workspace, everything but the data pointers filled in."""
+        key = (workspace.data_ptr(), workspace.stride(0), channel_count)
+        arr = self.arrays.get(key)
+        if arr is None:
+            if len(self.arrays) >= 16:
+                self.arrays.clear()
+            arr = (_Params * self.cp_size)()
+            max_ch = _device_max_channels(self.cp_size)
+            for r in range(self.cp_size):
+                p = arr[r]
+                for f in (p.send_fields[0], p.recv_fields[0]):
+                    f.element_count, f.element_size, f.stride_bytes = self.row0, self.elt, self.row0 * self.elt
+                for f in (p.send_fields[1], p.recv_fields[1]):
+                    f.element_count, f.element_size, f.stride_bytes = self.row1, 4, self.row1 * 4
+                p.entry_count = self.entries
+                p.workspace = key[0]
+                p.workspace_stride_u64 = key[1]
+                p.cp_rank, p.cp_size = r, self.cp_size
+                p.channel_count, p.max_channel_count = int(channel_count), max_ch
+            self.arrays[key] = arr
+        return arr
+
+
+_shapes: Dict[tuple, _ExchangeShape] = {}
+_call_lock = threading.RLock()  # the cached descriptor arrays are rewritten by every call
+
+
+def _exchange_shape(partial_o: torch.Tensor, softmax_stats: torch.Tensor, cp_size: int) -> _ExchangeShape:
+    """The cached facts of this pair's shape; the checks that depend on the tensors themselves run every time."""
+    _require(isinstance(partial_o, torch.Tensor) and isinstance(softmax_stats, torch.Tensor),
+             "partial_o and softmax_stats must be tensors")
+    key = (partial_o.shape, softmax_stats.shape, partial_o.dtype, softmax_stats.dtype, cp_size)
+    shape = _shapes.get(key)
+    if shape is None:
+        shape = _ExchangeShape(partial_o, softmax_stats, cp_size)
+        if len(_shapes) >= 256:
+            _shapes.clear()
+        _shapes[key] = shape
+        return shape
+    _require(partial_o.is_cuda, "partial_o must be on the GPU")
+    _require(softmax_stats.is_cuda, "softmax_stats must be on the GPU")
+    _require(partial_o.is_contiguous(), "partial_o must be contiguous")
+    _require(softmax_stats.is_contiguous(), "softmax_stats must be contiguous")
+    return shape
+
+
+def _env_channel_count() -> int:
+    """HELIX_A2A_CHANNEL_COUNT (csrc/torch_binding.cpp:25-32), 0 when unset or not a positive number."""
+    env = os.environ.get("HELIX_A2A_CHANNEL_COUNT")
+    if not env:
+        return 0
+    try:
+        n = int(env)
+    except ValueError:
+        return 0
+    return n if n > 0 else 0
+
+
+_PENDING_EXPIRY_S = 120.0  # a group that has waited this long for its last ranks is given up
+
+
+def set_pending_expiry(seconds: float) -> None:
+    """How long the first ranks of a per-rank exchange may wait for the last ones before the exchange is given up."""
+    global _PENDING_EXPIRY_S
+    _PENDING_EXPIRY_S = float(seconds)
 
 
 class _LogicalRankGroup:
@@ -258,51 +378,93 @@ class _LogicalRankGroup:
     every peer's send half, so it is enqueued when the last rank of the group
     has called: from then on stream order guarantees the lines are in the FIFOs.
     The tensors are kept alive here until that launch.
+
+    An exchange too large for the four FIFO entries of a stream cannot send
+    ahead of its receivers; its send halves are held back as well and the last
+    rank's call issues everything as one loopback exchange, which splits into
+    stream-ordered rounds (then a rank must leave its inputs alone until every
+    rank has called).
+
+    The channel count of an exchange (HELIX_A2A_CHANNEL_COUNT or automatic) is
+    settled by its first rank's call and used for every launch of it, whatever
+    the environment says later.
     """
 
     def __init__(self, cp_size: int) -> None:
         self.cp_size = cp_size
-        self.pending: Dict[int, Tuple[_Params, tuple, torch.cuda.Event, torch.cuda.Stream]] = {}
-        self.signature: Optional[tuple] = None
+        self.pending: Dict[int, Tuple[tuple, torch.cuda.Stream]] = {}
+        self.shape: Optional[_ExchangeShape] = None
+        self.arr: Optional[ctypes.Array] = None
+        self.deferred = False
+        self.started = 0.0
 
-    def submit(self, rank: int, params: _Params, keep: tuple, signature: tuple) -> None:
-        _require(rank not in self.pending,
-                 f"logical rank {rank} called alltoall again before all {self.cp_size} ranks of the group had called")
+    def _forget(self) -> None:
+        self.pending.clear()
+        self.shape = None
+        self.arr = None
+        self.deferred = False
+
+    def submit(self, rank: int, shape: _ExchangeShape, workspace: torch.Tensor, partial_o: torch.Tensor,
+               softmax_stats: torch.Tensor, out_o: torch.Tensor, out_s: torch.Tensor) -> None:
+        if self.pending and time.monotonic() - self.started > _PENDING_EXPIRY_S:
+            waited = sorted(self.pending)
+            self._forget()
+            raise RuntimeError(f"logical ranks {waited} waited more than {_PENDING_EXPIRY_S:.0f} s for the other ranks of "
+                               "their exchange; it is given up: re-initialise the workspace before the next exchange")
+        if rank in self.pending:
+            raise RuntimeError(f"logical rank {rank} called alltoall again before all {self.cp_size} ranks of the group had called")
         if self.pending:
-            _require(signature == self.signature, "logical ranks of one group must exchange tensors of one shape and dtype")
-        self.signature = signature
+            _require(shape is self.shape, "logical ranks of one group must exchange tensors of one shape and dtype")
+        else:
+            self.shape = shape
+            self.arr = shape.array(workspace, _env_channel_count())
+            self.deferred = False
+            self.started = time.monotonic()
+        p = self.arr[rank]
+        p.send_fields[0].data = partial_o.data_ptr()
+        p.send_fields[1].data = softmax_stats.data_ptr()
+        p.recv_fields[0].data = out_o.data_ptr()
+        p.recv_fields[1].data = out_s.data_ptr()
         stream = torch.cuda.current_stream()
-        _check(_lib.helix_a2a_alltoall_send(ctypes.byref(params), 1, stream.cuda_stream), "alltoall (send half)")
-        ev = torch.cuda.Event()
-        ev.record(stream)
-        self.pending[rank] = (params, keep, ev, stream)
+        if not self.deferred:
+            rc = _lib.helix_a2a_alltoall_send(ctypes.byref(p), 1, stream.cuda_stream)
+            if rc == 3 and not self.pending:  # HELIX_A2A_ERR_CAPACITY on the first rank: hold everything back
+                self.deferred = True
+            elif rc != 0:
+                if not self.pending:
+                    self._forget()
+                _raise_last("alltoall (send half)")
+        self.pending[rank] = ((partial_o, softmax_stats, out_o, out_s), stream)
         if len(self.pending) == self.cp_size:
-            self._flush()
+            self._flush(stream)
 
-    def _flush(self) -> None:
-        """Enqueue the receive half of every rank on the last caller's stream.
+    def _flush(self, stream: torch.cuda.Stream) -> None:
+        """Enqueue what is left of the exchange on the last caller's stream.
 
-        That stream first waits for every rank's send half; afterwards the
-        stream of every other rank waits for the receive launch, so each
-        rank's outputs are valid once the stream *it* called on has drained.
+        That stream first waits for the work of every other stream a rank called
+        on (its send half, or the producer of its inputs); afterwards those
+        streams wait for this launch, so each rank's outputs are valid once the
+        stream *it* called on has drained.
         """
-        arr = (_Params * self.cp_size)()
-        stream = torch.cuda.current_stream()
-        for r in range(self.cp_size):
-            params, _keep, ev, _rank_stream = self.pending[r]
-            arr[r] = params
-            stream.wait_event(ev)
+        others = {s.cuda_stream: s for _k, s in self.pending.values() if s.cuda_stream != stream.cuda_stream}
         try:
-            _check(_lib.helix_a2a_alltoall_recv(arr, self.cp_size, stream.cuda_stream), "alltoall (receive half)")
-            others = {s.cuda_stream: s for _p, _k, _e, s in self.pending.values() if s.cuda_stream != stream.cuda_stream}
+            for other in others.values():
+                ev = torch.cuda.Event()
+                ev.record(other)
+                stream.wait_event(ev)
+            if self.deferred:
+                rc = _lib.helix_a2a_alltoall_loopback(self.arr, self.cp_size, stream.cuda_stream)
+            else:
+                rc = _lib.helix_a2a_alltoall_recv(self.arr, self.cp_size, stream.cuda_stream)
+            if rc != 0:
+                _raise_last("alltoall (receive half)")
             if others:
                 done = torch.cuda.Event()
                 done.record(stream)
-                for s in others.values():
-                    s.wait_event(done)
+                for other in others.values():
+                    other.wait_event(done)
         finally:
-            self.pending.clear()
-            self.signature = None
+            self._forget()
 
 
 _groups: Dict[Tuple[int, int, int], _LogicalRankGroup] = {}
@@ -310,27 +472,33 @@ _groups: Dict[Tuple[int, int, int], _LogicalRankGroup] = {}
 
 def reset_logical_ranks() -> None:
     """Forget half-finished exchanges (e.g. after an error); the workspace must be re-initialised."""
-    _groups.clear()
+    with _call_lock:
+        _groups.clear()
+
+
+def _drop_group(key: Tuple[int, int, int]) -> None:
+    with _call_lock:
+        _groups.pop(key, None)
 
 
 def alltoall_native(partial_o: torch.Tensor, softmax_stats: torch.Tensor, workspace: torch.Tensor,
                     cp_rank: int, cp_size: int) -> Tuple[torch.Tensor, torch.Tensor]:
     """One logical rank's exchange; see :func:`helix_a2a.alltoall`."""
     _require(1 <= cp_size <= MAX_CP_SIZE, f"cp_size must be in [1, {MAX_CP_SIZE}]")
-    o3, s3 = _as_3d(partial_o, softmax_stats, cp_size)
+    shape = _exchange_shape(partial_o, softmax_stats, cp_size)
     _check_workspace(workspace, cp_size)
     _require(0 <= cp_rank < cp_size, "cp_rank must be in [0, cp_size)")
     _require(workspace.device == partial_o.device == softmax_stats.device, "all tensors must live on one device")
     out_o = torch.empty_like(partial_o)
     out_s = torch.empty_like(softmax_stats)
-    with torch.cuda.device(partial_o.device):
-        params = _make_params(o3, s3, out_o.view(o3.shape), out_s.view(s3.shape), workspace, cp_rank, cp_size, 0)
+    with _call_lock, _on_device(partial_o.device):
         key = (workspace.device.index or 0, workspace.data_ptr(), cp_size)
         group = _groups.get(key)
         if group is None:
             group = _groups[key] = _LogicalRankGroup(cp_size)
-        signature = (tuple(o3.shape), tuple(s3.shape), partial_o.dtype)
-        group.submit(cp_rank, params, (partial_o, softmax_stats, out_o, out_s, workspace), signature)
+            # nothing is left waiting on a workspace that no longer exists
+            weakref.finalize(workspace, _drop_group, key)
+        group.submit(cp_rank, shape, workspace, partial_o, softmax_stats, out_o, out_s)
     return out_o, out_s
 
 
@@ -343,27 +511,35 @@ def alltoall_loopback(partial_o: Sequence[torch.Tensor], softmax_stats: Sequence
     _require(1 <= cp_size <= MAX_CP_SIZE and len(softmax_stats) == cp_size,
              "need one partial_o and one softmax_stats tensor per rank")
     _check_workspace(workspace, cp_size)
-    arr = (_Params * cp_size)()
-    outs_o: List[torch.Tensor] = []
-    outs_s: List[torch.Tensor] = []
-    shape0 = None
-    with torch.cuda.device(workspace.device):
+    shape = _exchange_shape(partial_o[0], softmax_stats[0], cp_size)
+    device = workspace.device
+    if out is None:
+        # one allocation per field; rank r's result is slice r of it
+        outs_o = list(torch.empty((cp_size,) + tuple(shape.shape_o), dtype=shape.dtype, device=device).unbind(0))
+        outs_s = list(torch.empty((cp_size,) + tuple(shape.shape_s), dtype=torch.float32, device=device).unbind(0))
+    else:
+        outs_o, outs_s = list(out[0]), list(out[1])
+        _require(len(outs_o) == cp_size and len(outs_s) == cp_size, "need one output pair per rank")
+    with _call_lock, _on_device(device):
+        arr = shape.array(workspace, int(channel_count))
         for r in range(cp_size):
-            o3, s3 = _as_3d(partial_o[r], softmax_stats[r], cp_size)
-            sig = (tuple(o3.shape), tuple(s3.shape), partial_o[r].dtype)
-            shape0 = shape0 or sig
-            _require(sig == shape0, "all ranks must exchange tensors of one shape and dtype")
-            if out is None:
-                oo, os_ = torch.empty_like(partial_o[r]), torch.empty_like(softmax_stats[r])
-            else:
-                oo, os_ = out[0][r], out[1][r]
-                _require(oo.shape == partial_o[r].shape and oo.dtype == partial_o[r].dtype and oo.is_contiguous()
-                         and os_.shape == softmax_stats[r].shape and os_.dtype == torch.float32 and os_.is_contiguous()
+            o, st = partial_o[r], softmax_stats[r]
+            if r > 0:
+                _require(_exchange_shape(o, st, cp_size) is shape, "all ranks must exchange tensors of one shape and dtype")
+            _require(o.device == device and st.device == device, "all tensors must live on one device")
+            oo, os_ = outs_o[r], outs_s[r]
+            if out is not None:
+                _require(oo.shape == o.shape and oo.dtype == o.dtype and oo.is_contiguous()
+                         and os_.shape == st.shape and os_.dtype == torch.float32 and os_.is_contiguous()
                          and oo.is_cuda and os_.is_cuda, "out tensors must match the inputs")
-            outs_o.append(oo)
-            outs_s.append(os_)
-            arr[r] = _make_params(o3, s3, oo.view(o3.shape), os_.view(s3.shape), workspace, r, cp_size, channel_count)
-        _check(_lib.helix_a2a_alltoall_loopback(arr, cp_size, _stream_handle()), "alltoall_loopback")
+            p = arr[r]
+            p.send_fields[0].data = o.data_ptr()
+            p.send_fields[1].data = st.data_ptr()
+            p.recv_fields[0].data = oo.data_ptr()
+            p.recv_fields[1].data = os_.data_ptr()
+        rc = _lib.helix_a2a_alltoall_loopback(arr, cp_size, _stream_handle())
+    if rc != 0:
+        _raise_last("alltoall_loopback")
     return outs_o, outs_s
 
 
@@ -530,7 +706,7 @@ _reduce_lock = threading.Lock()  # the cached arrays are rewritten by every call
 
 
 def dcp_reduce(cp_attn_out: Sequence[torch.Tensor], cp_attn_lse: Sequence[torch.Tensor], workspace: torch.Tensor,
-               return_lse: bool, channel_count: int):
+               return_lse: bool, channel_count: int, lse_base2: bool = False):
     """Fused exchange + combine of ``[B, H, D]`` / ``[B, H]`` (natural-log LSE) per rank; see ``helix_a2a.dcp_a2a_lse_reduce``.
 
     Same kernel call as :class:`CombinePlan` with ``STATS_LSE_PACKED``; the
@@ -549,7 +725,6 @@ def dcp_reduce(cp_attn_out: Sequence[torch.Tensor], cp_attn_lse: Sequence[torch.
     _require(o0.is_cuda, "cp_attn_out must be on the GPU")
     _require(h % n == 0, "H must be divisible by the rank count")
     hp = h // n
-    _require(hp % 2 == 0, "H / N must be even (LSE rows are exchanged in 8-byte pieces)")
     _require(d % 4 == 0 and d >= 32, "head_dim must be a multiple of 4 and >= 32")
     _check_workspace(workspace, n)
     _require(workspace.device == device, "all tensors must live on one device")
@@ -563,7 +738,7 @@ def dcp_reduce(cp_attn_out: Sequence[torch.Tensor], cp_attn_lse: Sequence[torch.
     combined: List[torch.Tensor] = []
     lses: Optional[List[torch.Tensor]] = [] if return_lse else None
     keep = []
-    with _reduce_lock, torch.cuda.device(device):
+    with _reduce_lock, _on_device(device):
         for r in range(n):
             o, lse = cp_attn_out[r], cp_attn_lse[r]
             _require(o.shape == shape and o.dtype == dtype and o.device == device,
@@ -587,8 +762,8 @@ def dcp_reduce(cp_attn_out: Sequence[torch.Tensor], cp_attn_lse: Sequence[torch.
                 desc.out[r].lse_out = lo.data_ptr()
             else:
                 desc.out[r].lse_out = None
-        rc = _lib.helix_a2a_alltoall_combine_loopback(desc.arr, desc.out, n, STATS_LSE_PACKED, desc.dtype_code,
-                                                      _stream_handle())
+        mode = STATS_LSE_PACKED | (STATS_BASE2 if lse_base2 else 0)
+        rc = _lib.helix_a2a_alltoall_combine_loopback(desc.arr, desc.out, n, mode, desc.dtype_code, _stream_handle())
     if rc != 0:
         _raise_last("dcp_a2a_lse_reduce")
     return (combined, lses) if return_lse else combined

@@ -72,7 +72,7 @@ def wire_bytes(entries: int, field0_bytes: int, field1_bytes: int, cp: int, chan
     A stream (pair, channel) carries the entries ``channel, channel + channels, ...``; the messages it puts into
     one 1024-line FIFO entry form a run, stored piece after piece (8 bytes), 15 pieces + the flag word per line.
     """
-    pieces = (field0_bytes + field1_bytes) // 8
+    pieces = field0_bytes // 8 + -(-field1_bytes // 8)
     per_entry = 1024 * 15 // pieces
     lines = 0
     for ch in range(min(channels, entries)):

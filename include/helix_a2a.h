@@ -104,8 +104,11 @@ typedef struct helix_a2a_combine_out {
 /* how softmax_stats encodes the per-(entry, head) weight */
 #define HELIX_A2A_STATS_LSE 0     /* stats[2h] = natural-log LSE, stats[2h+1] ignored (patches/dcp_alltoall_helix.py:560-567) */
 #define HELIX_A2A_STATS_MAX_SUM 1 /* stats[2h] = running max, stats[2h+1] = running sum; LSE = max + ln(sum) */
-#define HELIX_A2A_STATS_LSE_PACKED 2 /* stats[h] = natural-log LSE of head h: the caller's [B, H] LSE tensor as it is
-                                        (patches/dcp_alltoall_helix.py:545-571 pads it to pairs only for the reference kernel) */
+#define HELIX_A2A_STATS_LSE_PACKED 2 /* stats[h] = natural-log LSE of head h: the caller's [B, H] LSE tensor as it is, any
+                                        number of heads per rank, rows 4-byte aligned (patches/dcp_alltoall_helix.py:545-571
+                                        pads it to pairs only for the reference kernel) */
+#define HELIX_A2A_STATS_BASE2 16     /* or-ed to one of the two LSE modes: the LSE values are base-2 logarithms, and lse_out is
+                                        written as one (is_lse_base_on_e = False, patches/dcp_alltoall_helix.py:183-186,199-203) */
 
 /* element type of partial_o for the combine arithmetic */
 #define HELIX_A2A_DTYPE_BF16 0
@@ -212,6 +215,7 @@ int helix_a2a_alltoall_loopback_static(const helix_a2a_params_t* per_rank, int c
  * Loopback exchange fused with the LSE-weighted combine: the receive half
  * reduces the cp_size partial outputs of each (entry, head) instead of storing
  * them. recv_fields of per_rank are ignored; out[r] receives rank r's result.
+ * stats_mode is one of HELIX_A2A_STATS_*, optionally or-ed with HELIX_A2A_STATS_BASE2.
  * heads = send_fields[1].element_count / 2 (element_count itself for HELIX_A2A_STATS_LSE_PACKED),
  * head_dim = send_fields[0].element_count / heads; head_dim must be a multiple of 4 and at least 32.
  */

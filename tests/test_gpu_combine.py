@@ -309,6 +309,49 @@ def test_dcp_a2a_lse_reduce_matches_the_reference_recipe(hx, ops, base_e):
         assert np.allclose(glse[r].cpu().numpy(), want_lse, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("n,h,d,base_e", [
+    (16, 16, 128, True),    # the 16-head MLA model of the reference's benchmark at N = 16: one head per rank
+    (4, 12, 64, True),      # three heads per rank
+    (4, 12, 64, False),     # ... with base-2 log-sum-exps
+    (8, 8, 576, False),     # one head per rank, MLA width (512 + 64), base 2
+    (2, 10, 32, True),      # five heads per rank, the smallest head
+    (3, 3, 96, True),       # one head per rank, three ranks
+])
+def test_dcp_a2a_lse_reduce_any_heads_per_rank(hx, ops, n, h, d, base_e):
+    # H/N need not be even: the reference pads every LSE to a pair (patches/dcp_alltoall_helix.py:560-567),
+    # here a row of H/N floats travels as it is; and the base of the logarithms is taken inside the kernel
+    b = 19
+    ws = workspace(hx, n)
+    g = torch.Generator().manual_seed(1000 * n + h)
+    outs = [torch.randn(b, h, d, generator=g).to(torch.bfloat16).cuda() for _ in range(n)]
+    lses = [(torch.randn(b, h, generator=g) * 3).cuda() for _ in range(n)]
+    lses[0][2, h - 1] = float("-inf")
+    lses[n - 1][b - 1, 0] = float("nan")
+    hp = h // n
+    o32 = np.stack([ho.bf16_bits_to_f32(torch_bits(t)) for t in outs])          # [N, B, H, D]
+    l32 = np.stack([t.cpu().numpy() for t in lses])                               # [N, B, H]
+    if not base_e:
+        l32 = l32 * np.float32(np.log(2.0))
+    for _ in range(2):   # the second call finds the descriptors of the shape cached
+        combined, glse = hx.dcp_a2a_lse_reduce(outs, lses, ws, return_lse=True, is_lse_base_on_e=base_e)
+        torch.cuda.synchronize()
+        assert ops.device_status() == 0
+        assert combined[0].shape == (b, hp, d) and glse[0].shape == (b, hp)
+        for r in range(n):
+            with np.errstate(all="ignore"):
+                want, want_lse = ho.lse_combine(o32[:, :, r * hp:(r + 1) * hp, :], l32[:, :, r * hp:(r + 1) * hp])
+            if not base_e:
+                want_lse = want_lse / np.float32(np.log(2.0))
+            got = combined[r].float().cpu().numpy()
+            assert (np.abs(got - want) <= ATOL + RTOL * np.abs(want)).all(), f"rank {r}"
+            assert np.allclose(glse[r].cpu().numpy(), want_lse, rtol=1e-4, atol=1e-4), f"rank {r}"
+    # without the combined LSE
+    only = hx.dcp_a2a_lse_reduce(outs, lses, ws, is_lse_base_on_e=base_e)
+    torch.cuda.synchronize()
+    for r in range(n):
+        assert torch.equal(only[r], combined[r])
+
+
 # ---------------------------------------------------------------------------
 # the pipeline benchmark's three formulations agree, eagerly and from captured graphs
 # ---------------------------------------------------------------------------
@@ -370,7 +413,6 @@ def test_dcp_a2a_lse_reduce_argument_checks_and_descriptor_reuse(hx, ops):
         (outs, [l.double() for l in lses], "float32"),
         (outs[:3] + [outs[3][:, :4]], lses, "one shape"),
         (make(hh=6)[0], make(hh=6)[1], "divisible"),
-        (make(hh=4)[0], make(hh=4)[1], "even"),                                     # one head per rank
         (make(dd=16)[0], make(dd=16)[1], "head_dim"),
     ]
     for o, l, pattern in bad:

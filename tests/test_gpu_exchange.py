@@ -2,6 +2,7 @@
 
 Bit-exact everywhere: the exchange moves opaque bytes.
 """
+import ctypes
 import os
 
 import numpy as np
@@ -630,13 +631,94 @@ def test_send_capacity_is_checked_for_split_phases(hx, ops):
     ws = get_workspace(hx, cp)
     o = torch.zeros(entries, cp, 64, dtype=torch.bfloat16, device="cuda")
     s = torch.zeros(entries, cp, 2, device="cuda")
+    oo, so = torch.empty_like(o), torch.empty_like(s)
+    p = ops._make_params(o, s, oo, so, ws, 0, cp, 1)
+    assert ops._lib.helix_a2a_alltoall_send(ctypes.byref(p), 1, ops._stream_handle()) == 3  # HELIX_A2A_ERR_CAPACITY
+    assert b"FIFO entries in flight" in ops._lib.helix_a2a_last_error()
+    assert ops._lib.helix_a2a_alltoall_recv(ctypes.byref(p), 1, ops._stream_handle()) == 3
+    torch.cuda.synchronize()
+    assert_clean(ops)
+
+
+def test_per_rank_calls_beyond_fifo_capacity(hx, ops):
+    # the reference accepts any entry count (its senders wait for their receivers); per-rank calls of logical
+    # ranks hold such an exchange back until the last rank has called and issue it in stream-ordered rounds
+    cp, entries = 3, 7300  # one channel: 3612 messages per round
+    ws = get_workspace(hx, cp)
+    g = torch.Generator().manual_seed(123)
+    ins_o = [torch.randint(-32768, 32767, (entries, cp, 64), generator=g, dtype=torch.int16).view(torch.bfloat16).cuda()
+             for _ in range(cp)]
+    ins_s = [torch.randint(-2**31, 2**31 - 1, (entries, cp, 2), generator=g, dtype=torch.int32).view(torch.float32).cuda()
+             for _ in range(cp)]
     os.environ["HELIX_A2A_CHANNEL_COUNT"] = "1"
     try:
-        with pytest.raises(RuntimeError, match="FIFO entries in flight"):
-            hx.alltoall(o, s, ws, 0, cp)
+        results = [hx.alltoall(ins_o[r], ins_s[r], ws, r, cp) for r in range(cp)]
     finally:
         del os.environ["HELIX_A2A_CHANNEL_COUNT"]
-    ops.reset_logical_ranks()
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(ins_o, ins_s, [x[0] for x in results], [x[1] for x in results], with_numpy=False)
+    # an exchange that fits goes back to sending at once, on the same workspace
+    small_o = [t[:100].contiguous() for t in ins_o]
+    small_s = [t[:100].contiguous() for t in ins_s]
+    results = [hx.alltoall(small_o[r], small_s[r], ws, r, cp) for r in range(cp)]
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(small_o, small_s, [x[0] for x in results], [x[1] for x in results], with_numpy=False)
+
+
+def test_channel_count_of_an_exchange_is_settled_by_its_first_rank(hx, ops):
+    # the send halves and the receive half of one per-rank exchange are separate launches; the environment
+    # may change between them without the halves disagreeing
+    cp, entries = 4, 40
+    ws = get_workspace(hx, cp)
+    g = torch.Generator().manual_seed(321)
+    ins_o = [torch.randint(-32768, 32767, (entries, cp, 128), generator=g, dtype=torch.int16).view(torch.bfloat16).cuda()
+             for _ in range(cp)]
+    ins_s = [torch.randint(-2**31, 2**31 - 1, (entries, cp, 4), generator=g, dtype=torch.int32).view(torch.float32).cuda()
+             for _ in range(cp)]
+    results = []
+    try:
+        for r in range(cp):
+            os.environ["HELIX_A2A_CHANNEL_COUNT"] = str(3 + 2 * r)
+            results.append(hx.alltoall(ins_o[r], ins_s[r], ws, r, cp))
+    finally:
+        del os.environ["HELIX_A2A_CHANNEL_COUNT"]
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(ins_o, ins_s, [x[0] for x in results], [x[1] for x in results], with_numpy=False)
+
+
+def test_abandoned_per_rank_exchange_expires(hx, ops):
+    # a group whose last ranks never call does not pin its tensors for ever: the next call after the expiry
+    # time gives the exchange up and says what to do
+    cp = 2
+    ws = get_workspace(hx, cp, fresh=True)
+    o = torch.zeros(4, cp, 64, dtype=torch.bfloat16, device="cuda")
+    s = torch.zeros(4, cp, 2, device="cuda")
+    ops.set_pending_expiry(0.0)
+    try:
+        hx.alltoall(o, s, ws, 0, cp)
+        with pytest.raises(RuntimeError, match="waited more than"):
+            hx.alltoall(o, s, ws, 0, cp)
+    finally:
+        ops.set_pending_expiry(120.0)
+    assert not any(g.pending for g in ops._groups.values())
+    torch.cuda.synchronize()
+    for r in range(cp):   # rank 0's lines sit in the FIFOs unreceived
+        hx.init_workspace(ws, r, cp)
+    # a workspace that goes away takes its group along
+    ws2 = hx.allocate_workspace(cp, 0)
+    for r in range(cp):
+        hx.init_workspace(ws2, r, cp)
+    hx.alltoall(o, s, ws2, 0, cp)
+    key = (ws2.device.index or 0, ws2.data_ptr(), cp)
+    assert key in ops._groups
+    torch.cuda.synchronize()
+    del ws2
+    import gc
+    gc.collect()
+    assert key not in ops._groups
 
 
 @pytest.mark.parametrize("single_round", [False, True])
