@@ -26,6 +26,23 @@ def build_host_model() -> Path:
     return HOST_MODEL_LIB
 
 
+C_ABI_HOST_SRC = ROOT / "tests" / "c_abi" / "gpu_host.c"
+C_ABI_HOST_EXE = ROOT / "tests" / "c_abi" / "gpu_host"
+
+
+def build_c_abi_host() -> Path:
+    """Compile tests/c_abi/gpu_host.c as C99 against include/helix_a2a.h, the library and the HIP runtime."""
+    rocm = Path("/opt/rocm")
+    cmd = ["gcc", "-std=c99", "-O1", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__", f"-I{rocm / 'include'}",
+           f"-I{ROOT / 'include'}", str(C_ABI_HOST_SRC), "-o", str(C_ABI_HOST_EXE),
+           f"-L{ROOT / 'helix-a2a_amd' / 'helix_a2a'}", "-lhelix_a2a", f"-L{rocm / 'lib'}", "-lamdhip64",
+           "-Wl,-rpath,$ORIGIN/../../helix-a2a_amd/helix_a2a", f"-Wl,-rpath,{rocm / 'lib'}"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("building the C host failed:\n" + proc.stdout + proc.stderr)
+    return C_ABI_HOST_EXE
+
+
 class _Field(ctypes.Structure):
     _fields_ = [("data", ctypes.c_void_p), ("element_count", ctypes.c_int32),
                 ("element_size", ctypes.c_int32), ("stride_bytes", ctypes.c_int32)]

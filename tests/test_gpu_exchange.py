@@ -421,6 +421,41 @@ def test_many_calls_back_to_back_without_sync(hx, ops):
     assert int(bad.item()) == 0
 
 
+def test_exchange_beside_a_competing_kernel(hx, ops):
+    # Sender wavefronts come first in a launch's dispatch order, and receivers rely on that to find their
+    # senders running. Here the device is shared with long unrelated kernels on a second stream of the same
+    # (default) priority, which take wavefront slots away from the exchange at arbitrary moments: the
+    # exchanges must still complete, bit for bit, with no wait running into its limit.
+    from helix_a2a.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS["c3"]
+    ws = get_workspace(hx, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    want_o, want_s = expected_on_device(ins_o), expected_on_device(ins_s)
+    side = torch.cuda.Stream()
+    noise = torch.randn(1 << 26, device="cuda")             # 256 MB: every launch fills the device for a while
+    small = torch.randn(1 << 16, device="cuda")             # and short ones in between
+    bad = torch.zeros((), dtype=torch.int64, device="cuda")
+    torch.cuda.synchronize()
+    plan = ops.LoopbackPlan(ins_o, ins_s, ws)
+    for it in range(40):
+        with torch.cuda.stream(side):
+            noise.mul_(1.0001).sin_()
+            for _ in range(4):
+                small.add_(1.0)
+        outs_o, outs_s = plan.run()
+        for r in range(w.cp):
+            bad += (outs_o[r].view(torch.int16) != want_o[r].view(torch.int16)).sum()
+            bad += (outs_s[r].view(torch.int32) != want_s[r].view(torch.int32)).sum()
+        if it % 10 == 9:
+            torch.cuda.synchronize()
+            assert ops.device_status() == 0, f"a wait gave up in iterations {it - 9}..{it}"
+            assert int(bad.item()) == 0, f"wrong output in iterations {it - 9}..{it}"
+    side.synchronize()
+    torch.cuda.synchronize()
+    assert ops.device_status() == 0 and int(bad.item()) == 0
+
+
 # ---------------------------------------------------------------------------
 # the per-rank call (the reference's signature)
 # ---------------------------------------------------------------------------
@@ -851,6 +886,20 @@ def test_single_rank_call_both_halves(hx, ops):
 # ---------------------------------------------------------------------------
 # nothing to exchange: zero entries is a valid call that launches nothing
 # ---------------------------------------------------------------------------
+
+def test_plain_c_host_drives_the_exchange(hx, ops):
+    # tests/c_abi/gpu_host.c: hipMalloc + include/helix_a2a.h, no torch -- what a native binding would do
+    import subprocess
+
+    from helix_testing import C_ABI_HOST_EXE
+
+    assert C_ABI_HOST_EXE.exists(), "build it with __graft_entry__.build() (tests/helix_testing.py::build_c_abi_host)"
+    torch.cuda.synchronize()
+    run = subprocess.run([str(C_ABI_HOST_EXE)], capture_output=True, text=True, timeout=100)
+    assert run.returncode == 0 and "gpu_host ok" in run.stdout, run.stdout + run.stderr
+    for what in ("loopback:", "loopback again:", "send halves + receive half:", "loopback through the built-in workspace:"):
+        assert f"{what} 0 wrong element(s)" in run.stdout, run.stdout
+
 
 def test_empty_inputs(hx, ops):
     cp = 4
