@@ -152,6 +152,31 @@ def host_timing(w, ws, ins_o, ins_s, calls: int = 200):
     return out
 
 
+def cold_only(args, w, make_plan, ins_o, ins_s, bytes_per_call) -> int:
+    """The cold leg alone: every step on the next of N sets of tensors; prints a short JSON line."""
+    import torch
+
+    from helix_a2a import _ops
+
+    tensor_bytes = sum(t.numel() * t.element_size() for t in ins_o + ins_s) * 2
+    n_sets = args.rotate if args.rotate >= 2 else max(2, -(-(1 << 30) // tensor_bytes))
+    plans = [make_plan([t.clone() for t in ins_o], [t.clone() for t in ins_s]) for _ in range(n_sets)]
+    for i in range(max(args.warmup, n_sets)):
+        plans[i % n_sets].run()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for i in range(args.steps):
+        plans[i % n_sets].run()
+    end.record()
+    torch.cuda.synchronize()
+    status = _ops.device_status()
+    us = start.elapsed_time(end) / args.steps * 1e3
+    print(json.dumps({"workload": w.name, "leg": "cold", "sets": n_sets, "kernel_us": us,
+                      "frac_cold": bytes_per_call / (us * 1e-6) / 1e9 / PEAK_HBM_GBPS, "status": status}))
+    return 0 if status == 0 else 1
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -169,6 +194,9 @@ def main() -> int:
                     help="sets of input and output tensors the cold leg cycles through (every step takes the next "
                          "set, so the working set exceeds the 256 MB memory-side cache); -1 = as many as make "
                          "1 GiB of tensors, 0 = no cold leg")
+    ap.add_argument("--cold-only", action="store_true",
+                    help="run only the cold leg (warm-up and timed steps over the rotating sets): for profiler runs "
+                         "that must not mix launches of the two legs")
     ap.add_argument("--units-per-wavefront", type=int, default=None, metavar="U",
                     help="share runs longer than U KiB per wavefront between wavefronts (library default: 6; 0 = never)")
     ap.add_argument("--no-host-timing", action="store_true", help="skip the host-time-per-call measurements")
@@ -221,6 +249,8 @@ def main() -> int:
     wire = w.run_wire_bytes(channels, per_head)
     bytes_per_call = w.combine_bytes(channels) if args.combine else w.exchange_bytes(channels, per_head)
 
+    if args.cold_only:
+        return cold_only(args, w, make_plan, ins_o, ins_s, bytes_per_call)
     for _ in range(args.warmup):
         plan.run()
     torch.cuda.synchronize()

@@ -535,6 +535,7 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, cons
   a.lseBase2 = base2 ? 1 : 0;
   a.dtype = dtype;
   a.headMagic = head_div_magic(static_cast<uint32_t>(a.headDim) * 2u / kPieceBytes);
+  a.np0Magic = div_magic(static_cast<uint32_t>(plan.shape.np0));
   const uint64_t outBytes = static_cast<uint64_t>(plan.entryCount) * a.field0Bytes;
   if (outBytes >= 2147483648ull) return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "combined output exceeds 2 GiB");
   a.recvBytes0 = static_cast<uint32_t>(outBytes);
@@ -553,11 +554,12 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, cons
     a.entryBegin = begin;
     long end = static_cast<long>(begin) + plan.roundEntries;
     a.entryEnd = end > plan.entryCount ? plan.entryCount : static_cast<int>(end);
-    // wavefronts per (receiver, channel): enough to cover a round's units once, and to fill the device
+    // wavefronts per (receiver, channel): enough to cover a round's output pieces once, and to fill the device
     int msgs = stream_msg_count(a.entryBegin, a.entryEnd, 0, a.runChannels);
     int perEntry = msgs_per_fifo_entry(plan.shape);
-    long runUnits = run_units(msgs < perEntry ? msgs : perEntry, plan.shape);
-    long cover = (runUnits + kWaveLanes - 1) / kWaveLanes;
+    long runPieces = static_cast<long>(msgs < perEntry ? msgs : perEntry) * plan.shape.np0;
+    long perTurn = (cp_size <= 8 ? 2 : 1) * kWaveLanes;  // pieces a wavefront takes per turn
+    long cover = (runPieces + perTurn - 1) / perTurn;
     long fill = static_cast<long>(plan.cuCount) * 16 / (static_cast<long>(cp_size) * a.runChannels);
     long parts = cover < fill ? cover : fill;
     if (parts < 1) parts = 1;

@@ -561,60 +561,50 @@ __device__ __forceinline__ void widen4<1>(u32x2 piece, float (&f)[4]) {  // fp16
   f[3] = __half2float(__ushort_as_half(static_cast<unsigned short>(piece.y >> 16)));
 }
 
-template <int kDtype>
-__device__ __forceinline__ uint32_t narrow1(float v);
-template <>
-__device__ __forceinline__ uint32_t narrow1<0>(float v) {  // fp32 -> bf16, round to nearest even, NaN stays NaN
-  uint32_t b = __float_as_uint(v);
-  if ((b & 0x7FFFFFFFu) > 0x7F800000u) return (b >> 16) | 0x0040u;
-  return (b + 0x7FFFu + ((b >> 16) & 1u)) >> 16;
-}
-template <>
-__device__ __forceinline__ uint32_t narrow1<1>(float v) {
-  return static_cast<uint32_t>(__half_as_ushort(__float2half_rn(v)));
-}
-
-// Receive half of the fused form. A wavefront serves one (receiver, channel)
-// and all cpSize senders at once: lane L owns run unit U (the same unit of
-// the same message in every sender's FIFO, since all streams of a channel
-// share one layout), loads that unit from each sender's FIFO, and reduces
-// over the senders in registers:
+// Receive half of the fused form. The workgroup of one (receiver, channel) walks the payload of the
+// run in output order: its wavefronts take turns at accesses of 64 consecutive 8-byte pieces of the
+// combined output, a lane owns one piece (four elements of one head of one entry), finds that piece
+// in the run (message j, piece p -> run piece j*np + p -> line and word: the same place in every
+// sender's FIFO, since all streams of a channel share one layout), loads it from each sender's
+// FIFO, and reduces over the senders in registers:
 //   out[e, h, :] = sum_s w[s, h] * partial_o_s[e, h, :],  w = softmax_s(lse[s, h])
-// (patches/dcp_alltoall_helix.py:142-207). The wavefront first acquires the
-// run from every sender through the head token, so every line it touches
-// afterwards is complete.
+// (patches/dcp_alltoall_helix.py:142-207). The output goes out as one coalesced 8-byte store per
+// lane. The wavefront first acquires the run from every sender through that sender's step counter,
+// so every line it touches afterwards is complete (the flag words are not loaded here at all).
 //
-// Weights are computed once per wavefront and (message, head), not once per
-// lane: the 64 units of a wave access cover a handful of heads. The lanes that
-// start a head enter it in a slot table (LDS), then the wavefront turns
-// sideways -- lane j serves slot j / G and sender j % G, loads that sender's
-// statistics of that head, and a softmax over the G lanes of a slot gives
-// the weight -- and the weights go back through LDS to the lanes that own
-// units of the head. (G = 4, 8, 16 or 32 lanes per slot for cpSize <= 4, 8, 16, 32.)
-// The `parts` wavefronts of a workgroup split the units of a run.
-constexpr int kCombineSlots = 32;  // distinct (message, head) pairs one wave access may touch
+// Weights are computed once per wavefront and (message, head), not once per lane: the pieces of an
+// access cover a few heads. The lanes that start a head enter it in a slot table (LDS), then the
+// wavefront turns sideways -- lane i serves slot i / G and sender i % G, loads that sender's
+// statistics of that head, and a softmax over the G lanes of a slot gives the weight -- and the
+// weights go back through LDS to the lanes that own pieces of the head. (G = 4, 8, 16 or 32 lanes
+// per slot for cpSize <= 4, 8, 16, 32.) With up to eight senders a lane handles two accesses per
+// turn, so that sixteen loads are in flight either way.
+constexpr int kCombineSlots = 32;  // distinct (message, head) pairs one turn may touch (head_dim >= 32: at most 18)
 
 struct CombineCtx {
   __amdgpu_buffer_rsrc_t fifos;  // the whole FIFO region of the receiver's row
   uint32_t channelBase;          // byte offset of sender 0's FIFO of this channel
   uint32_t senderStride;         // bytes between the FIFOs of consecutive senders
-  uint32_t stepLo, stepHi;       // lane q: step counter of sender q's stream
+  uint32_t stepLo;               // lane q: step counter (low word) of sender q's stream
 };
 
 template <int kLanesPerSlot>
 struct CombineLds {
-  uint32_t slot[kMaxCombineParts][kCombineSlots][4];          // {first run piece of the message, head, entry, -}
-  float weight[kMaxCombineParts][kCombineSlots][kLanesPerSlot];  // normalised softmax weight per sender
+  uint32_t slot[kMaxCombineParts][kCombineSlots][4];  // {first run piece of the message, head, entry, -}
+  float __attribute__((aligned(16))) weight[kMaxCombineParts][kCombineSlots][kLanesPerSlot];  // softmax weight per sender
 };
 
-__device__ __forceinline__ uint32_t shuffle_from(uint32_t v, int srcLane) {
-  return static_cast<uint32_t>(__shfl(static_cast<int>(v), srcLane, kWaveLanes));
-}
 __device__ __forceinline__ float shuffle_xor(float v, int mask) { return __shfl_xor(v, mask, kWaveLanes); }
 
 // byte offset of sender q's open FIFO entry inside the receiver's FIFO region
 __device__ __forceinline__ uint32_t entry_base(const CombineCtx& cx, int q, uint32_t stepLo) {
   return cx.channelBase + static_cast<uint32_t>(q) * cx.senderStride + (stepLo & (kFifoDepth - 1)) * kFifoEntryBytes;
+}
+
+// byte offset of run piece g inside a FIFO entry: line g / 15, word g % 15
+__device__ __forceinline__ uint32_t run_piece_offset(uint32_t g) {
+  const uint32_t line = __umulhi(g, 0x11111112u);  // floor(g / 15) for g < 2^16 (div_magic(15))
+  return line * kLineBytes + (g - line * kPiecesPerLine) * kPieceBytes;
 }
 
 // exp and ln on the hardware's base-2 units (v_exp_f32 / v_log_f32, about 1 ulp):
@@ -636,10 +626,25 @@ __device__ __forceinline__ float lse_of_stats(uint32_t s0, uint32_t s1, int stat
   return (isnan(x) || isinf(x)) ? -INFINITY : x;
 }
 
+// four fp32 -> one 8-byte piece of bf16 (v_cvt_pk_bf16_f32: round to nearest even, NaN stays NaN) or fp16
 template <int kDtype>
-__device__ __forceinline__ u32x2 narrow_piece(const float (&acc)[4]) {
-  u32x2 r = {narrow1<kDtype>(acc[0]) | (narrow1<kDtype>(acc[1]) << 16),
-             narrow1<kDtype>(acc[2]) | (narrow1<kDtype>(acc[3]) << 16)};
+__device__ __forceinline__ u32x2 narrow_piece(const float (&acc)[4]);
+template <>
+__device__ __forceinline__ u32x2 narrow_piece<0>(const float (&acc)[4]) {
+  using f32x2 = float __attribute__((ext_vector_type(2)));
+  using bf16x2 = __bf16 __attribute__((ext_vector_type(2)));
+  const bf16x2 lo = __builtin_convertvector(f32x2{acc[0], acc[1]}, bf16x2);
+  const bf16x2 hi = __builtin_convertvector(f32x2{acc[2], acc[3]}, bf16x2);
+  u32x2 r = {__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi)};
+  return r;
+}
+template <>
+__device__ __forceinline__ u32x2 narrow_piece<1>(const float (&acc)[4]) {
+  using f32x2 = float __attribute__((ext_vector_type(2)));
+  using f16x2 = _Float16 __attribute__((ext_vector_type(2)));
+  const f16x2 lo = __builtin_convertvector(f32x2{acc[0], acc[1]}, f16x2);  // round to nearest even
+  const f16x2 hi = __builtin_convertvector(f32x2{acc[2], acc[3]}, f16x2);
+  u32x2 r = {__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi)};
   return r;
 }
 
@@ -648,6 +653,8 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
                                                      int lane, CombineLds<kLanesPerSlot>& lds, int probe) {
   HELIX_MARK(probe, 0, false);
   constexpr int kSlotsPerPass = kWaveLanes / kLanesPerSlot;
+  constexpr int kAccesses = kLanesPerSlot <= 8 ? 2 : 1;                  // accesses a lane handles per turn
+  constexpr int kGroup = kLanesPerSlot <= 16 ? kLanesPerSlot : 16;       // senders whose pieces are in flight together
   Stream st;
   setup_stream(st, a, 0, ch);
   if (st.msgs == 0) return;  // uniform over the workgroup: same channel
@@ -658,7 +665,8 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
   cx.senderStride = static_cast<uint32_t>(fifo_offset(1, 0, a.maxChannels));
   __amdgpu_buffer_rsrc_t outRsrc = make_rsrc(a.rank[r].recv0, a.recvBytes0);
   __amdgpu_buffer_rsrc_t lseRsrc = make_rsrc(a.rank[r].recv1, a.rank[r].recv1 ? a.recvBytes1 : 0u);
-  const unsigned long long lanesBelow = (1ull << lane) - 1ull;
+  const unsigned long long lanesUpToMe = (2ull << lane) - 1ull;  // lanes 0..lane
+  const uint32_t piecesPerHead = static_cast<uint32_t>(a.headDim) / 4u;
 
   // lane q owns the counters of sender q's stream
   int64_t myStep = 0;
@@ -687,13 +695,12 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
 
   for (int firstMsg = 0; firstMsg < st.msgs; firstMsg += st.msgsPerEntry, myStep += 1) {
     const int runMsgs = min(st.msgsPerEntry, st.msgs - firstMsg);
-    const uint32_t runUnits = stream_run_units(st, runMsgs);
+    const uint32_t runPieces = static_cast<uint32_t>(runMsgs) * st.np0;  // payload pieces of the run = output pieces
     cx.stepLo = static_cast<uint32_t>(myStep);
-    cx.stepHi = static_cast<uint32_t>(static_cast<uint64_t>(myStep) >> 32);
     {
-      // Acquire the run from every sender: a head beyond the step says that all
+      // Acquire the run from every sender: a counter beyond the step says that all
       // lines of the step are in memory (the sender waits for its stores before
-      // it moves head). Every unit needs all cpSize senders anyway.
+      // it moves it). Every piece needs all cpSize senders anyway.
       SpinGuard guard(a.spinLimitTicks, broken_word(a));
       for (;;) {
         const bool closed = lane >= a.cpSize || ld_counter(&mySenderInfo[0]) > myStep;
@@ -707,83 +714,77 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
       asm volatile("" ::: "memory");
     }
     if (firstMsg == 0) HELIX_MARK(probe, 1, false);
-    for (uint32_t U0 = static_cast<uint32_t>(part) * kWaveLanes; U0 < runUnits;
-         U0 += static_cast<uint32_t>(parts) * kWaveLanes) {
-      const uint32_t U = U0 + lane;
-      const RunUnit d = decode_run_unit(U, st.np, st.npMagic);
-      const bool live = U < runUnits;
-      const bool dataA = live && d.msgA < static_cast<uint32_t>(runMsgs) && d.pieceA < st.np0;
-      const bool dataB = live && !d.flag && d.msgB < static_cast<uint32_t>(runMsgs) && d.pieceB < st.np0;
-      if (__ballot(dataA || dataB) == 0ull) continue;  // statistics, padding: nothing to reduce here
-      const uint32_t hA = head_of_piece(d.pieceA, a.headMagic);
-      const uint32_t hB = head_of_piece(d.pieceB, a.headMagic);
-      const uint32_t pairA = d.msgA * static_cast<uint32_t>(a.heads) + hA;
-      const uint32_t pairB = d.msgB * static_cast<uint32_t>(a.heads) + hB;
-      const bool ownB = dataB && (!dataA || pairB != pairA);  // the second piece starts the next head (or message)
-      const uint32_t entryA = static_cast<uint32_t>(a.entryBegin + ch) + (firstMsg + d.msgA) * a.runChannels;
-      const uint32_t entryB = static_cast<uint32_t>(a.entryBegin + ch) + (firstMsg + d.msgB) * a.runChannels;
-
-      // Up to eight senders: their unit loads go out before the weights are
-      // worked out -- they do not depend on them, and the two round trips
-      // overlap. (With sixteen, holding the first eight units that long costs a
-      // quarter of the resident wavefronts, which costs more than it saves.)
-      // Senders beyond cpSize are read out of range (zeros, no memory traffic),
-      // which keeps the sequence free of branches.
-      constexpr bool kLoadUnitsEarly = kLanesPerSlot <= 8;
-      u32x4 v[8];
-      auto load_units = [&](int g) {
+    for (uint32_t P0 = static_cast<uint32_t>(part) * (kAccesses * kWaveLanes); P0 < runPieces;
+         P0 += static_cast<uint32_t>(parts) * (kAccesses * kWaveLanes)) {
+      // ---- where this lane's pieces are: in the run (every sender's FIFO alike) and in the output
+      bool live[kAccesses];
+      uint32_t fifoOff[kAccesses], outOff[kAccesses], msg[kAccesses], head[kAccesses], entry[kAccesses], piece[kAccesses];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int q = g + j;
-          if (q < kLanesPerSlot) {
-            const int qs = q < a.cpSize ? q : 0;
-            const uint32_t off = entry_base(cx, qs, lane_value(cx.stepLo, qs)) + U * kUnitBytes;
-            v[j] = __builtin_amdgcn_raw_buffer_load_b128(cx.fifos, (live && q < a.cpSize) ? off : kOutOfRange, 0, kAuxSc1);
-          }
+      for (int k = 0; k < kAccesses; ++k) {
+        const uint32_t P = P0 + static_cast<uint32_t>(k) * kWaveLanes + lane;
+        live[k] = P < runPieces;
+        msg[k] = div_by_magic(P, a.np0Magic);
+        piece[k] = P - msg[k] * st.np0;
+        head[k] = head_of_piece(piece[k], a.headMagic);
+        entry[k] = static_cast<uint32_t>(a.entryBegin + ch) + (firstMsg + msg[k]) * a.runChannels;
+        fifoOff[k] = live[k] ? run_piece_offset(msg[k] * st.np + piece[k]) : kOutOfRange;
+        outOff[k] = live[k] ? (entry[k] * st.np0 + piece[k]) * kPieceBytes : kOutOfRange;
+      }
+
+      // The pieces do not depend on the weights: their loads go out first, and that round trip
+      // overlaps the one of the statistics. Senders beyond cpSize are read out of range (zeros, no
+      // memory traffic), which keeps the sequence free of branches.
+      u32x2 v[kAccesses][kGroup];
+      auto load_group = [&](int g) {
+#pragma unroll
+        for (int jq = 0; jq < kGroup; ++jq) {
+          const int q = g + jq;
+          const int qs = q < a.cpSize ? q : 0;
+          const uint32_t base = entry_base(cx, qs, lane_value(cx.stepLo, qs));
+#pragma unroll
+          for (int k = 0; k < kAccesses; ++k)
+            v[k][jq] = __builtin_amdgcn_raw_buffer_load_b64(cx.fifos, q < a.cpSize ? base + fifoOff[k] : kOutOfRange, 0, kAuxSc1);
         }
       };
-      if (kLoadUnitsEarly) load_units(0);
+      load_group(0);
 
-      // ---- slots: one per distinct (message, head) the lanes of this access touch, in lane order
-      const uint32_t lastPair = dataB ? pairB : (dataA ? pairA : 0xFFFFFFFFu);
-      const uint32_t prevPair = shuffle_from(lastPair, lane == 0 ? 0 : lane - 1);
-      const bool newA = dataA && (lane == 0 || prevPair != pairA);
-      const unsigned long long startsA = __ballot(newA), startsB = __ballot(ownB);
-      const int slotA = __popcll(startsA & (lanesBelow | (1ull << lane))) + __popcll(startsB & lanesBelow) - 1;
-      const int slotB = ownB ? slotA + 1 : slotA;
-      const int slotCount = __popcll(startsA) + __popcll(startsB);
+      // ---- slots: one per distinct (message, head) the lanes of this turn touch, in piece order
+      int mySlot[kAccesses];
+      int slotCount = 0;
+#pragma unroll
+      for (int k = 0; k < kAccesses; ++k) {
+        const bool starts = live[k] && (lane == 0 || piece[k] == head[k] * piecesPerHead);
+        const unsigned long long mask = __ballot(starts);
+        mySlot[k] = slotCount + __popcll(mask & lanesUpToMe) - 1;
+        if (starts) {
+          lds.slot[part][mySlot[k]][0] = msg[k] * st.np;
+          lds.slot[part][mySlot[k]][1] = head[k];
+          lds.slot[part][mySlot[k]][2] = entry[k];
+        }
+        if (!live[k]) mySlot[k] = 0;
+        slotCount += __popcll(mask);
+      }
       if (slotCount > kCombineSlots) {  // excluded by the host's shape check (head_dim >= 32)
         raise_status(a, kStatusInternal, lane);
         return;
-      }
-      if (newA) {
-        lds.slot[part][slotA][0] = d.msgA * st.np;
-        lds.slot[part][slotA][1] = hA;
-        lds.slot[part][slotA][2] = entryA;
-      }
-      if (ownB) {
-        lds.slot[part][slotB][0] = d.msgB * st.np;
-        lds.slot[part][slotB][1] = hB;
-        lds.slot[part][slotB][2] = entryB;
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-      // ---- weights: lane j serves slot base + j / G and sender j % G
+      // ---- weights: lane i serves slot base + i / G and sender i % G
       for (int base = 0; base < slotCount; base += kSlotsPerPass) {
         const int slot = base + lane / kLanesPerSlot;
         const int q = lane % kLanesPerSlot;
-        const bool serving = slot < slotCount && q < a.cpSize;
-        const int slotSafe = slot < kCombineSlots ? slot : 0;
+        const bool inSlot = slot < slotCount;
+        const bool serving = inSlot && q < a.cpSize;
+        const int slotSafe = inSlot ? slot : 0;
         const uint32_t msgPiece0 = lds.slot[part][slotSafe][0];
         const uint32_t h = lds.slot[part][slotSafe][1];
         const uint32_t slotEntry = lds.slot[part][slotSafe][2];
         const uint32_t gs = msgPiece0 + st.np0 + (a.statsMode == 2 ? h >> 1 : h);  // run piece that holds head h's statistics
-        const uint32_t ls = gs / kPiecesPerLine;
-        const uint32_t word = gs - ls * kPiecesPerLine;
-        const uint32_t qStepLo = shuffle_from(cx.stepLo, q < a.cpSize ? q : 0);
-        const uint32_t off = entry_base(cx, q, qStepLo) + ls * kLineBytes + word * kPieceBytes;
+        const uint32_t qStepLo = static_cast<uint32_t>(__shfl(static_cast<int>(cx.stepLo), q < a.cpSize ? q : 0, kWaveLanes));
+        const uint32_t off = entry_base(cx, q, qStepLo) + run_piece_offset(gs);
         const u32x2 sv = __builtin_amdgcn_raw_buffer_load_b64(cx.fifos, serving ? off : kOutOfRange, 0, kAuxSc1);
         const float lse = serving ? lse_of_stats(sv.x, sv.y, a.statsMode, h, a.lseBase2 != 0) : -INFINITY;
         float m = lse;
@@ -795,7 +796,8 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
         float total = e;
 #pragma unroll
         for (int x = 1; x < kLanesPerSlot; x <<= 1) total += shuffle_xor(total, x);
-        if (serving) lds.weight[part][slotSafe][q] = e / fmaxf(total, 1e-10f);
+        // (senders beyond cpSize get weight 0: their pieces are read as zeros, and 0 * 0 stays 0)
+        if (inSlot) lds.weight[part][slotSafe][q] = e * __builtin_amdgcn_rcpf(fmaxf(total, 1e-10f));
         // one lane per slot reports the head's combined log-sum-exp
         const float combinedLse = fast_log(total) + m;
         __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(a.lseBase2 ? combinedLse * 1.4426950408889634f : combinedLse), lseRsrc,
@@ -806,46 +808,32 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-      // ---- the unit of every sender, weighted
-      const float* wA = lds.weight[part][dataA ? slotA : 0];
-      const float* wB = lds.weight[part][dataB ? slotB : 0];
-      float accA[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-      float accB[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-      uint32_t flagMismatch = 0u;
-#pragma unroll 1  // sixteen senders: one group of eight units in registers at a time
-      for (int g = 0; g < kLanesPerSlot; g += 8) {
-        if (g > 0 || !kLoadUnitsEarly) load_units(g);
+      // ---- the piece of every sender, weighted
+      float acc[kAccesses][4];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int q = g + j;
-          if (q < kLanesPerSlot) {
-            const bool have = q < a.cpSize;
-            const int qs = have ? q : 0;
-            const float wa = have ? wA[q] : 0.0f, wb = have ? wB[q] : 0.0f;
+      for (int k = 0; k < kAccesses; ++k)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[k][c] = 0.0f;
+#pragma unroll 1  // thirty-two senders: one group of sixteen pieces in registers at a time
+      for (int g = 0; g < kLanesPerSlot; g += kGroup) {
+        if (g > 0) load_group(g);
+#pragma unroll
+        for (int k = 0; k < kAccesses; ++k) {
+          const float* w = &lds.weight[part][mySlot[k]][g];
+#pragma unroll
+          for (int jq = 0; jq < kGroup; ++jq) {
             float f[4];
-            u32x2 pa = {v[j].x, v[j].y};
-            u32x2 pb = {v[j].z, v[j].w};
-            widen4<kDtype>(pa, f);
+            widen4<kDtype>(v[k][jq], f);
+            const float wq = w[jq];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) accA[c] += wa * f[c];
-            widen4<kDtype>(pb, f);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) accB[c] += wb * f[c];
-            if (live && d.flag && have)
-              flagMismatch |= (v[j].z ^ lane_value(cx.stepLo, qs)) | (v[j].w ^ lane_value(cx.stepHi, qs));
+            for (int c = 0; c < 4; ++c) acc[k][c] += wq * f[c];
           }
         }
       }
-      if (__ballot(flagMismatch != 0u) != 0ull) {
-        // the head tokens promised complete lines: a flag that disagrees means the workspace is corrupt
-        raise_status(a, kStatusInternal, lane);
-        return;
-      }
-      __builtin_amdgcn_raw_buffer_store_b64(narrow_piece<kDtype>(accA), outRsrc,
-                                            dataA ? (entryA * st.np0 + d.pieceA) * kPieceBytes : kOutOfRange, 0, kAuxNone);
-      __builtin_amdgcn_raw_buffer_store_b64(narrow_piece<kDtype>(accB), outRsrc,
-                                            dataB ? (entryB * st.np0 + d.pieceB) * kPieceBytes : kOutOfRange, 0, kAuxNone);
-      __builtin_amdgcn_wave_barrier();  // the tables are rewritten by the next access
+#pragma unroll
+      for (int k = 0; k < kAccesses; ++k)
+        __builtin_amdgcn_raw_buffer_store_b64(narrow_piece<kDtype>(acc[k]), outRsrc, outOff[k], 0, kAuxNone);
+      __builtin_amdgcn_wave_barrier();  // the tables are rewritten by the next turn
     }
   }
   HELIX_MARK(probe, 2, false);

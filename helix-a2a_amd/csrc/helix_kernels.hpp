@@ -45,6 +45,7 @@ struct KernelArgs {
   int statsMode, dtype;
   int lseBase2;        // the statistics are base-2 logarithms, and so is the combined log-sum-exp that is stored
   uint32_t headMagic;  // head_div_magic(pieces per head)
+  uint32_t np0Magic;   // div_magic(pieces of field 0)
 };
 
 // Wavefronts of a workgroup are independent (no LDS, no barrier); small
