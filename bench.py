@@ -152,6 +152,45 @@ def host_timing(w, ws, ins_o, ins_s, calls: int = 200):
     return out
 
 
+def copy_calibration(mib: int) -> None:
+    """Five launches of a plain elementwise kernel that reads exactly ``mib`` MiB and writes exactly ``mib`` MiB:
+    what a counter run scales FETCH_SIZE and WRITE_SIZE by."""
+    import torch
+
+    n = mib * (1 << 20) // 4
+    src = torch.arange(n, dtype=torch.int32, device="cuda")
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for _ in range(5):
+        torch.add(src, 1, out=dst)  # one kernel: reads 4n bytes, writes 4n bytes
+    torch.cuda.synchronize()
+
+
+def memory_probe(mib: int = 1024, reps: int = 20):
+    """What plain kernels reach on this box, for scale: an elementwise copy (reads and writes ``mib`` MiB,
+    beyond the memory-side cache) and a fill (writes only), in GB/s of bytes moved."""
+    import torch
+
+    n = mib * (1 << 20) // 4
+    src = torch.arange(n, dtype=torch.int32, device="cuda")
+    dst = torch.empty_like(src)
+    out = {}
+    for name, fn, moved in (("copy_GBps", lambda: torch.add(src, 1, out=dst), 8 * n), ("fill_GBps", lambda: dst.fill_(7), 4 * n)):
+        for _ in range(3):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        out[name] = moved / (a.elapsed_time(b) * 1e-3 / reps) / 1e9
+    out["note"] = (f"torch elementwise kernels on {mib} MiB tensors: copy = read + write of the same size, fill = write only; "
+                   "a yardstick for what mixed and write-only traffic reach on this box, not a roofline")
+    return out
+
+
 def cold_only(args, w, make_plan, ins_o, ins_s, bytes_per_call) -> int:
     """The cold leg alone: every step on the next of N sets of tensors; prints a short JSON line."""
     import torch
@@ -172,6 +211,8 @@ def cold_only(args, w, make_plan, ins_o, ins_s, bytes_per_call) -> int:
     torch.cuda.synchronize()
     status = _ops.device_status()
     us = start.elapsed_time(end) / args.steps * 1e3
+    if args.copy_calibration:
+        copy_calibration(args.copy_calibration)
     print(json.dumps({"workload": w.name, "leg": "cold", "sets": n_sets, "kernel_us": us,
                       "frac_cold": bytes_per_call / (us * 1e-6) / 1e9 / PEAK_HBM_GBPS, "status": status}))
     return 0 if status == 0 else 1
@@ -347,13 +388,7 @@ def main() -> int:
             ok &= torch.equal(outs_s[r].view(torch.int32), want_s[r].view(torch.int32))
 
     if args.copy_calibration:
-        n = args.copy_calibration * (1 << 20) // 4
-        src = torch.arange(n, dtype=torch.int32, device="cuda")
-        dst = torch.empty_like(src)
-        torch.cuda.synchronize()
-        for _ in range(5):
-            torch.add(src, 1, out=dst)  # one kernel: reads 4n bytes, writes 4n bytes
-        torch.cuda.synchronize()
+        copy_calibration(args.copy_calibration)
 
     achieved = bytes_per_call / (avg_kernel_ms * 1e-3) / 1e9
     kernel_name = "helix_combine_kernel" if args.combine else "helix_exchange_kernel"
@@ -418,6 +453,7 @@ def main() -> int:
     }
     if not args.no_host_timing and not args.combine and args.layout == "token" and graph is None:
         result["host_us_per_call"] = host_timing(w, ws, ins_o, ins_s)
+        result["memory_probe"] = memory_probe()
     if not args.no_cpu_baseline and not args.combine and args.layout == "token":
         result["cpu_baseline"] = cpu_baseline(w, bytes_per_call)
     print(json.dumps(result))

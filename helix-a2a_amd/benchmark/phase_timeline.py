@@ -116,6 +116,16 @@ def main() -> int:
             col = allrows[:, k]
             print(f"| {kind} | {names[kind][k]} | {pct(col, 0.05):.2f} | {pct(col, 0.5):.2f} | {pct(col, 0.95):.2f} | {col.max():.2f} |")
     print()
+    print("when wavefronts start and finish: share of all wavefronts per microsecond since the first start")
+    allrows = np.concatenate(rows["send"] + rows["recv"], axis=0)
+    top = int(np.ceil(allrows[:, 3].max()))
+    width = max(1, top // 24)
+    print("| us | " + " | ".join(f"{lo}-{lo + width}" for lo in range(0, top, width)) + " |")
+    print("|---|" + "---|" * len(range(0, top, width)))
+    for label, col in (("started", 0), ("done", 3)):
+        hist, _ = np.histogram(allrows[:, col], bins=list(range(0, top + width, width)))
+        print(f"| {label} | " + " | ".join(f"{100.0 * h / allrows.shape[0]:.0f} %" for h in hist[:len(range(0, top, width))]) + " |")
+    print()
     print("time between consecutive points of one wavefront (us)")
     print("| wavefronts | interval | p5 | p50 | p95 |")
     print("|---|---|---|---|---|")

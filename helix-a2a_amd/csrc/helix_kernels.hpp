@@ -48,10 +48,10 @@ struct KernelArgs {
   uint32_t np0Magic;   // div_magic(pieces of field 0)
 };
 
-// Wavefronts of a workgroup are independent (no LDS, no barrier); small
-// workgroups dispatch and retire at a finer grain (2 measured best of 1..16).
+// Wavefronts of a workgroup of the exchange kernel are independent (no LDS, no barrier); small
+// workgroups dispatch and retire at a finer grain (2 measured best of 1..16 on launches that queue).
 constexpr int kWavesPerBlock = 2;
-constexpr int kBlockThreads = kWavesPerBlock * kWaveLanes;
+constexpr int kResidentWavefronts = 4096;  // 256 CUs x 4 SIMDs x 4 wavefronts: what runs at once
 
 // streams one direction of a launch serves: one per (local rank, channel, peer)
 inline int waves_per_direction(const KernelArgs& a) { return a.rankCount * a.runChannels * a.cpSize; }
