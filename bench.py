@@ -6,10 +6,14 @@
 One step = one loopback exchange of all cp logical ranks of the workload
 (payload read + FIFO write + FIFO read + output write), inputs resident in HBM.
 Prints ONE JSON line: effective GB/s (algorithmic bytes / time per call) and
-microseconds per call, the roofline fraction of the exchange kernel (measured
-with HIP events on the launch stream) and a CPU baseline (the reference tests'
-torch transpose recipe and the C restatement of the reference kernel, timed on
-this machine's host cores).
+microseconds per call; the roofline fraction of the kernel measured with HIP
+events on the launch stream, once with one set of tensors reused every step
+(`roofline.frac`; at c3 that working set fits the 256 MB memory-side cache) and
+once over rotating sets of tensors (`roofline.frac_cold`); the rate of payload
+alone; the host time of the drop-in calls; what plain copy and fill kernels
+reach on the same box; and a CPU baseline (the reference tests' torch
+transpose recipe and the C restatement of the reference kernel, timed on this
+machine's host cores).
 """
 from __future__ import annotations
 
@@ -32,10 +36,15 @@ PEAK_HBM_GBPS = 8000.0
 # Bytes that crossed between the L2s and the fabric per launch (FETCH_SIZE + WRITE_SIZE of two
 # rocprofv3 --pmc runs, each scaled by the same counter of a plain copy kernel), one row per profiled
 # configuration: (kernel, workload, channels) -> bytes. The summaries under profiles/ named
-# <kernel>_<workload>_hbm_traffic.md hold the runs these come from. These counters sit between L2
-# and fabric: they do not tell whether the memory-side cache or DRAM served a request.
+# <kernel>_<workload>.md hold the runs these come from. These counters sit between L2 and fabric:
+# they do not tell whether the memory-side cache or DRAM served a request.
 MEASURED_TRAFFIC_BYTES = {
-    ("helix_exchange_kernel", "c3", 128): 150_201_931,
+    ("helix_exchange_kernel", "c3", 128): 150_760_007,   # profiles/helix_exchange_kernel_c3.md
+    ("helix_exchange_kernel", "c4", 128): 566_408_454,   # profiles/helix_exchange_kernel_c4.md
+    ("helix_exchange_kernel", "c5a", 64): 600_359_122,   # profiles/helix_exchange_kernel_c5a.md
+    ("helix_combine_kernel", "c3", 128): 118_961_054,    # profiles/helix_combine_kernel_c3.md
+    ("helix_combine_kernel", "c4", 128): 451_869_515,    # profiles/helix_combine_kernel_c4.md
+    ("helix_combine_kernel", "c5a", 64): 464_350_556,    # profiles/helix_combine_kernel_c5a.md
 }
 
 
