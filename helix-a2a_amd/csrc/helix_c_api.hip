@@ -55,6 +55,7 @@ bool checked_mode() {
 // -1 = kMaxUnitsInFlight, and only while the launch leaves wavefront slots of the device free;
 // 0 = never share; 1..6 = always share beyond that many.
 std::atomic<int> g_unitsPerWavefront{-1};
+std::atomic<int> g_teamUnits{-1};
 
 // Wavefronts per stream a launch may use at most. The automatic rule looks at the whole exchange (both
 // directions of all cp ranks), not at the launch, so that the send and receive halves of one exchange
@@ -65,6 +66,8 @@ int max_parts_for(const KernelArgs& a, int cuCount) {
   if (mode > 0) return kMaxStreamParts;
   return auto_max_parts(a.cpSize, a.runChannels, cuCount);
 }
+int team_units() { return g_teamUnits.load(); }
+
 int units_per_part() {
   const int mode = g_unitsPerWavefront.load();
   return mode > 0 ? mode : kMaxUnitsInFlight;
@@ -350,14 +353,14 @@ int launch_rounds(Plan& plan, bool send, bool recv, bool allowRounds, hipStream_
     long waves = 2L * waves_per_direction(a);
     if (waves > static_cast<long>(plan.cuCount) * 8)
       return fail(HELIX_A2A_ERR_CAPACITY, "single-round launch of %ld wavefronts is not guaranteed co-resident", waves);
-    HELIX_HIP_TRY(launch_exchange(a, kMaxUnitsInFlight, 1, stream));  // senders wait on the one tail counter: one wavefront per stream
+    HELIX_HIP_TRY(launch_exchange(a, kMaxUnitsInFlight, 1, 0, stream));  // senders wait on the one tail counter: one wavefront per stream
     return HELIX_A2A_OK;
   }
   for (int begin = 0; begin < plan.entryCount; begin += plan.roundEntries) {
     a.entryBegin = begin;
     long end = static_cast<long>(begin) + plan.roundEntries;
     a.entryEnd = end > plan.entryCount ? plan.entryCount : static_cast<int>(end);
-    HELIX_HIP_TRY(launch_exchange(a, units_per_part(), max_parts_for(a, plan.cuCount), stream));
+    HELIX_HIP_TRY(launch_exchange(a, units_per_part(), max_parts_for(a, plan.cuCount), team_units(), stream));
   }
   return HELIX_A2A_OK;
 }
@@ -585,6 +588,13 @@ void helix_a2a_set_spin_limit_us(uint64_t microseconds) { g_spinLimitUs.store(mi
 
 void helix_a2a_set_single_round(int enabled) { g_singleRound.store(enabled ? 1 : 0); }
 
+
+int helix_a2a_set_team_units(int units) {
+  if (units < -1 || units > kMaxUnitsInFlight)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "units per team wavefront must be in [-1, %d], got %d", kMaxUnitsInFlight, units);
+  g_teamUnits.store(units);
+  return HELIX_A2A_OK;
+}
 
 int helix_a2a_set_units_per_wavefront(int units) {
   if (units < -1 || units > kMaxUnitsInFlight)

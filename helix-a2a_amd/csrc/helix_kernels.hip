@@ -167,6 +167,38 @@ __device__ __forceinline__ void report_broken(const KernelArgs& a, int lane) {
   if (lane == 0) atomicOr(a.status, kStatusBrokenWorkspace);
 }
 
+// A team: the wavefronts of one workgroup that walk one stream's run together, each a slice of it. Only
+// the first wavefront (the leader) touches the stream's counters; it hands the step (or -1: give up) to
+// the others through this word of LDS. Launches whose wavefronts queue for slots anyway use teams for
+// runs of several passes: the same bytes move in more, shorter wavefronts without one more counter.
+struct TeamLds {
+  int64_t step;
+};
+// A barrier of the workgroup that waits for this wavefront's LDS traffic only (not, as __syncthreads
+// does, for its outstanding loads and stores to memory).
+__device__ __forceinline__ void team_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// The leader's step, or -1, for every wavefront of the team.
+__device__ __forceinline__ int64_t team_share_step(TeamLds* lds, bool leader, int lane, int64_t step) {
+  if (leader && lane == 0) *reinterpret_cast<volatile int64_t*>(&lds->step) = step;
+  team_barrier();
+  return *reinterpret_cast<volatile int64_t*>(&lds->step);
+}
+
+// Every scalar of the argument block a wavefront needs before its first memory access, asked for at once:
+// the compiler then fetches the block in a few wide scalar loads and one wait at the top of the kernel,
+// instead of one small load and one wait wherever a field is first used (a dozen dependent trips to the
+// scalar cache before the first payload load otherwise).
+__device__ __forceinline__ void fetch_scalars_up_front(const KernelArgs& a) {
+  asm volatile("" ::"s"(a.workspace), "s"(a.rowStrideBytes), "s"(a.cpSize), "s"(a.maxChannels), "s"(a.runChannels),
+               "s"(a.entryBegin), "s"(a.field0Bytes), "s"(a.field1Bytes), "s"(a.sendStride0), "s"(a.sendStride1),
+               "s"(a.recvStride0), "s"(a.recvStride1), "s"(a.sendBytes0), "s"(a.sendBytes1), "s"(a.recvBytes0),
+               "s"(a.recvBytes1), "s"(a.npMagic), "s"(a.rankBegin), "s"(a.rankCount), "s"(a.doSend), "s"(a.doRecv));
+  asm volatile("" ::"s"(a.parts), "s"(a.team), "s"(a.np0), "s"(a.np), "s"(a.msgsPerEntry), "s"(a.baseMsgs),
+               "s"(a.extraChannels), "s"(a.byParts.magic), "s"(a.byParts.shift), "s"(a.byTeam.magic), "s"(a.byTeam.shift),
+               "s"(a.byCp.magic), "s"(a.byCp.shift), "s"(a.byChannels.magic), "s"(a.byChannels.shift), "s"(a.sendBlocks), "s"(a.wavesPerBlock),
+               "s"(a.spinLimitTicks));
+}
+
 // What a stream's wavefront needs to know, all wave-uniform.
 struct Stream {
   __amdgpu_buffer_rsrc_t fifo;    // the 512 KiB FIFO of the stream
@@ -181,12 +213,11 @@ struct Stream {
 };
 
 __device__ __forceinline__ void setup_stream(Stream& st, const KernelArgs& a, int peer, int ch) {
-  const MsgShape sh = make_msg_shape(a.field0Bytes, a.field1Bytes);
-  st.np0 = sh.np0;
-  st.np = sh.np;
+  st.np0 = static_cast<uint32_t>(a.np0);
+  st.np = static_cast<uint32_t>(a.np);
   st.npMagic = a.npMagic;
-  st.msgsPerEntry = msgs_per_fifo_entry(sh);
-  st.msgs = stream_msg_count(a.entryBegin, a.entryEnd, ch, a.runChannels);
+  st.msgsPerEntry = a.msgsPerEntry;
+  st.msgs = a.baseMsgs + (ch < a.extraChannels ? 1 : 0);  // stream_msg_count(a.entryBegin, a.entryEnd, ch, a.runChannels)
   st.firstRow = static_cast<uint32_t>(a.entryBegin + ch) * a.cpSize + peer;
   st.rowStep = static_cast<uint32_t>(a.runChannels) * a.cpSize;
 }
@@ -229,16 +260,20 @@ __device__ __forceinline__ UnitOffsets unit_offsets(const Stream& st, uint32_t f
 // sender
 // ---------------------------------------------------------------------------
 // Part `part` of the a.parts wavefronts that send stream (s -> r, ch): it walks its slice of every run.
-template <int kAux, int kUnitsInFlight>
-__device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, int ch, int part, int lane, int wave) {
+// With kTeam the parts are the a.team wavefronts of this workgroup and share part 0's counters.
+template <int kAux, int kUnitsInFlight, bool kTeam = false>
+__device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, int ch, int part, int lane, int wave,
+                                           TeamLds* lds = nullptr) {
   HELIX_MARK(wave, 0, false);
+  const bool leader = !kTeam || part == 0;
+  const int sliceCount = kTeam ? a.team : a.parts;
   Stream st;
   setup_stream(st, a, r, ch);
   if (st.msgs == 0) return;
   uint8_t* senderRow = a.workspace + static_cast<uint64_t>(s) * a.rowStrideBytes;
   uint8_t* receiverRow = a.workspace + static_cast<uint64_t>(r) * a.rowStrideBytes;
   int64_t* info = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(a.cpSize, a.maxChannels, r, ch));
-  int64_t* token = info + sender_counter_slot(part);
+  int64_t* token = info + sender_counter_slot(kTeam ? 0 : part);
   st.fifo = make_rsrc(receiverRow + fifo_offset(s, ch, a.maxChannels), kFifoBytes);
   st.field0 = make_rsrc(a.rank[s].send0, a.sendBytes0);
   st.field1 = make_rsrc(a.rank[s].send1, a.sendBytes1);
@@ -246,25 +281,28 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
   st.stride1 = a.sendStride1;
 
   // the counters are only needed once the first payload loads are in flight
-  int64_t step = *token;
-  int64_t tail = info[1];
-  const uint64_t broken = broken_at_launch(a);
+  int64_t step = 0, tail = 0;
+  uint64_t broken = 0;
+  if (leader) {
+    step = *token;
+    tail = info[1];
+    broken = broken_at_launch(a);
+  }
 
   for (int firstMsg = 0; firstMsg < st.msgs; firstMsg += st.msgsPerEntry) {
     const int runMsgs = min(st.msgsPerEntry, st.msgs - firstMsg);
     const uint32_t runUnits = stream_run_units(st, runMsgs);
-    const Slice slice = slice_of_run(runUnits, part, a.parts);
+    const Slice slice = slice_of_run(runUnits, part, sliceCount, kTeam ? a.byTeam : a.byParts);
     bool opened = false;
     // open the FIFO entry of this run (csrc/helix_alltoall.cu:377-390); false when the wait for room gave up
-    auto open_entry = [&]() -> bool {
-      opened = true;
+    auto leader_opens = [&]() -> bool {
       if (broken != 0) {
         report_broken(a, lane);
         return false;
       }
       if (firstMsg > 0) {
         step += 1;
-        wait_stores_acknowledged();
+        if (!kTeam) wait_stores_acknowledged();
         if (lane == 0) st_counter(token, step);
       }
       SpinGuard guard(a.spinLimitTicks, broken_word(a));
@@ -278,6 +316,18 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
         __builtin_amdgcn_s_sleep(4);
       }
       return true;
+    };
+    auto open_entry = [&]() -> bool {
+      opened = true;
+      if (!kTeam) return leader_opens();
+      if (firstMsg > 0) {  // the leader closes the previous entry once every wavefront's lines of it are in memory
+        wait_stores_acknowledged();
+        team_barrier();
+      }
+      bool ok = true;
+      if (leader) ok = leader_opens();
+      step = team_share_step(lds, leader, lane, ok ? step : -1);
+      return step >= 0;
     };
     for (uint32_t U0 = slice.begin; U0 < slice.end; U0 += kUnitsInFlight * kWaveLanes) {
       u32x2 wa[kUnitsInFlight], wb[kUnitsInFlight];
@@ -343,7 +393,8 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
   HELIX_MARK(wave, 2, false);
   wait_stores_acknowledged();
   HELIX_MARK(wave, 3, false);
-  if (lane == 0) st_counter(token, step + 1);
+  if (kTeam) team_barrier();
+  if (leader && lane == 0) st_counter(token, step + 1);
 }
 
 // ---------------------------------------------------------------------------
@@ -353,9 +404,13 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
 // part (that part's counter beyond the step: all its lines of the step are in memory), reads its slice
 // in passes of kUnitsInFlight units per lane and stores the payload. Line flags are still compared: one
 // that disagrees after the token means the workspace is corrupt.
-template <int kAux, int kUnitsInFlight, bool kAlignedStores>
-__device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, int ch, int part, int lane, int wave) {
+template <int kAux, int kUnitsInFlight, bool kAlignedStores, bool kTeam = false>
+__device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, int ch, int part, int lane, int wave,
+                                             TeamLds* lds = nullptr) {
   HELIX_MARK(wave, 0, false);
+  const bool leader = !kTeam || part == 0;
+  const int sliceCount = kTeam ? a.team : a.parts;
+  const int counterPart = kTeam ? 0 : part;
   Stream st;
   setup_stream(st, a, s, ch);
   if (st.msgs == 0) return;
@@ -363,45 +418,63 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
   uint8_t* receiverRow = a.workspace + static_cast<uint64_t>(r) * a.rowStrideBytes;
   int64_t* senderInfo = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(a.cpSize, a.maxChannels, r, ch));
   int64_t* info = reinterpret_cast<int64_t*>(receiverRow + receiver_info_offset(a.cpSize, a.maxChannels, s, ch));
-  int64_t* token = senderInfo + sender_counter_slot(part);
-  int64_t* mine = info + receiver_counter_slot(part);
+  int64_t* token = senderInfo + sender_counter_slot(counterPart);
+  int64_t* mine = info + receiver_counter_slot(counterPart);
   st.fifo = make_rsrc(receiverRow + fifo_offset(s, ch, a.maxChannels), kFifoBytes);
   st.field0 = make_rsrc(a.rank[r].recv0, a.recvBytes0);
   st.field1 = make_rsrc(a.rank[r].recv1, a.recvBytes1);
   st.stride0 = a.recvStride0;
   st.stride1 = a.recvStride1;
 
-  int64_t step = *mine;
-  int64_t head = ld_counter(token);
-  if (broken_at_launch(a) != 0) {
-    report_broken(a, lane);
-    return;
+  int64_t step = 0, head = 0;
+  bool broken = false;
+  if (leader) {
+    step = *mine;
+    head = ld_counter(token);
+    broken = broken_at_launch(a) != 0;
   }
 
   for (int firstMsg = 0; firstMsg < st.msgs; firstMsg += st.msgsPerEntry) {
     const int runMsgs = min(st.msgsPerEntry, st.msgs - firstMsg);
     const uint32_t runUnits = stream_run_units(st, runMsgs);
-    const Slice slice = slice_of_run(runUnits, part, a.parts);
-    if (firstMsg > 0) {
-      // this part's lines of the previous entry have been consumed (csrc/helix_alltoall.cu:427-449);
-      // part 0's counter is the tail the sender's back-pressure reads
-      step += 1;
-      if (lane == 0) {
-        st_counter(mine, step);
-        if (part == 0) st_counter(&senderInfo[1], step);
+    const Slice slice = slice_of_run(runUnits, part, sliceCount, kTeam ? a.byTeam : a.byParts);
+    // the leader releases the previous entry and waits for the token of this one; false when it gave up
+    auto leader_acquires = [&]() -> bool {
+      if (broken) {
+        report_broken(a, lane);
+        return false;
       }
-    }
-    if (head <= step) {
-      SpinGuard guard(a.spinLimitTicks, broken_word(a));
-      for (;;) {
-        head = ld_counter(token);
-        if (head > step) break;
-        if (guard.expired()) {
-          raise_status(a, kStatusRecvTimeout, lane);
-          return;
+      if (firstMsg > 0) {
+        // the lines of the previous entry have been consumed (csrc/helix_alltoall.cu:427-449);
+        // part 0's counter is the tail the sender's back-pressure reads
+        step += 1;
+        if (lane == 0) {
+          st_counter(mine, step);
+          if (counterPart == 0) st_counter(&senderInfo[1], step);
         }
-        __builtin_amdgcn_s_sleep(1);
       }
+      if (head <= step) {
+        SpinGuard guard(a.spinLimitTicks, broken_word(a));
+        for (;;) {
+          head = ld_counter(token);
+          if (head > step) break;
+          if (guard.expired()) {
+            raise_status(a, kStatusRecvTimeout, lane);
+            return false;
+          }
+          __builtin_amdgcn_s_sleep(1);
+        }
+      }
+      return true;
+    };
+    if (!kTeam) {
+      if (!leader_acquires()) return;
+    } else {
+      if (firstMsg > 0) team_barrier();  // every wavefront of the team has its lines of the previous entry in registers
+      bool ok = true;
+      if (leader) ok = leader_acquires();
+      step = team_share_step(lds, leader, lane, ok ? step : -1);
+      if (step < 0) return;
     }
     asm volatile("" ::: "memory");  // no line is read before the token was seen
     const uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
@@ -492,9 +565,10 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
     }
   }
   HELIX_MARK(wave, 2, false);
-  if (lane == 0) {  // close the last entry (csrc/helix_alltoall.cu:468-472)
+  if (kTeam) team_barrier();  // every wavefront of the team has the lines of the last entry in registers
+  if (leader && lane == 0) {  // close the last entry (csrc/helix_alltoall.cu:468-472)
     st_counter(mine, step + 1);
-    if (part == 0) st_counter(&senderInfo[1], step + 1);
+    if (counterPart == 0) st_counter(&senderInfo[1], step + 1);
   }
   HELIX_MARK(wave, 3, true);
 }
@@ -515,28 +589,32 @@ __device__ __forceinline__ void run_sender_any(const KernelArgs& a, int s, int r
 // that no receiver can occupy a slot a not-yet-started sender needs.
 // Within a direction, w = ((local rank * runChannels + channel) * cp + peer) * parts + part:
 // neighbouring wavefronts touch neighbouring slices, then neighbouring rows of the same entry.
-template <int kUnitsInFlight, bool kAlignedStores>
+// With kTeam a workgroup is one team: workgroup b serves stream b of the launch (parts = 1).
+template <int kUnitsInFlight, bool kAlignedStores, bool kTeam>
 __global__ __launch_bounds__(1024) HELIX_WAVES_PER_SIMD void helix_exchange_kernel(KernelArgs a) {
+  __shared__ TeamLds teamLds;
+  fetch_scalars_up_front(a);
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWaveLanes);
   const int lane = static_cast<int>(threadIdx.x) % kWaveLanes;
-  int w = static_cast<int>(blockIdx.x) * (static_cast<int>(blockDim.x) / kWaveLanes) + wave;
-  const int probe = w;  // index of this wavefront's phase stamps (a stamped build only)
+  const int probe = static_cast<int>(blockIdx.x) * a.wavesPerBlock + wave;  // index of the wavefront in the launch
+  int w = kTeam ? static_cast<int>(blockIdx.x) : probe;
   const int perDirection = a.rankCount * a.runChannels * a.cpSize * a.parts;
   const int senders = a.doSend ? perDirection : 0;
   const int total = senders + (a.doRecv ? perDirection : 0);
   if (w >= total) return;
   const bool isSender = w < senders;
   if (!isSender) w -= senders;
-  const int part = w % a.parts;
-  const int q = w / a.parts;
-  const int peer = q % a.cpSize;
-  const int t = q / a.cpSize;
-  const int ch = t % a.runChannels;
-  const int local = a.rankBegin + t / a.runChannels;
+  const int q = static_cast<int>(fast_div_by(static_cast<uint32_t>(w), a.byParts));
+  const int part = kTeam ? wave : w - q * a.parts;
+  const int t = static_cast<int>(fast_div_by(static_cast<uint32_t>(q), a.byCp));
+  const int peer = q - t * a.cpSize;
+  const int localIndex = static_cast<int>(fast_div_by(static_cast<uint32_t>(t), a.byChannels));
+  const int ch = t - localIndex * a.runChannels;
+  const int local = a.rankBegin + localIndex;
   if (isSender) {
-    run_sender<kAuxSc1, kUnitsInFlight>(a, local, peer, ch, part, lane, probe);
+    run_sender<kAuxSc1, kUnitsInFlight, kTeam>(a, local, peer, ch, part, lane, probe, &teamLds);
   } else {
-    run_receiver<kAuxSc1, kUnitsInFlight, kAlignedStores>(a, local, peer, ch, part, lane, probe);
+    run_receiver<kAuxSc1, kUnitsInFlight, kAlignedStores, kTeam>(a, local, peer, ch, part, lane, probe, &teamLds);
   }
 }
 
@@ -687,8 +765,7 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
   if (part == 0 && lane < a.cpSize) {
     // rounds never put more than the four entries in flight, so the entries can
     // be handed back up front; nothing reads these counters before the launch ends
-    const MsgShape sh = make_msg_shape(a.field0Bytes, a.field1Bytes);
-    int64_t done = myStep + entries_for_msgs(st.msgs, sh);
+    int64_t done = myStep + (ch < a.extraChannels ? a.entriesExtra : a.entriesBase);  // entries_for_msgs(st.msgs)
     st_counter(&myInfo[1], done);
     st_counter(&mySenderInfo[1], done);
   }
@@ -846,22 +923,25 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
 template <int kDtype, int kLanesPerSlot>
 __global__ __launch_bounds__(kMaxCombineParts * kWaveLanes) HELIX_WAVES_PER_SIMD void helix_combine_kernel(KernelArgs a) {
   __shared__ CombineLds<kLanesPerSlot> lds;
-  const int parts = static_cast<int>(blockDim.x) / kWaveLanes;
+  fetch_scalars_up_front(a);
+  const int parts = a.wavesPerBlock;
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWaveLanes);
   const int lane = static_cast<int>(threadIdx.x) % kWaveLanes;
   const int senderStreams = a.doSend ? a.rankCount * a.runChannels * a.cpSize : 0;
-  const int sendBlocks = (senderStreams + parts - 1) / parts;
+  const int sendBlocks = a.doSend ? a.sendBlocks : 0;  // ceil(senderStreams / parts)
   int b = static_cast<int>(blockIdx.x);
   if (b < sendBlocks) {
     const int w = b * parts + wave;
     if (w >= senderStreams) return;
-    const int t = w / a.cpSize;
-    run_sender_any<kAuxSc1>(a, a.rankBegin + t / a.runChannels, w % a.cpSize, t % a.runChannels, 0, lane, w);
+    const int t = static_cast<int>(fast_div_by(static_cast<uint32_t>(w), a.byCp));
+    const int localIndex = static_cast<int>(fast_div_by(static_cast<uint32_t>(t), a.byChannels));
+    run_sender_any<kAuxSc1>(a, a.rankBegin + localIndex, w - t * a.cpSize, t - localIndex * a.runChannels, 0, lane, w);
     return;
   }
   b -= sendBlocks;
-  const int r = a.rankBegin + b / a.runChannels;
-  const int ch = b % a.runChannels;
+  const int localIndex = static_cast<int>(fast_div_by(static_cast<uint32_t>(b), a.byChannels));
+  const int r = a.rankBegin + localIndex;
+  const int ch = b - localIndex * a.runChannels;
   run_combine_receiver<kDtype, kLanesPerSlot>(a, r, ch, wave, parts, lane, lds, senderStreams + b * parts + wave);
 }
 
@@ -908,30 +988,69 @@ static long largest_run_units(const KernelArgs& a) {
   return run_units(msgs < perEntry ? msgs : perEntry, sh);
 }
 
-hipError_t launch_exchange(const KernelArgs& args, int unitsPerPart, int maxParts, hipStream_t stream) {
+// The fields of the argument block that follow from the others (see KernelArgs); a.parts and a.team are set.
+static void set_launch_constants(KernelArgs& a) {
+  const MsgShape sh = make_msg_shape(a.field0Bytes, a.field1Bytes);
+  a.np0 = sh.np0;
+  a.np = sh.np;
+  a.msgsPerEntry = msgs_per_fifo_entry(sh);
+  const int entries = a.entryEnd > a.entryBegin ? a.entryEnd - a.entryBegin : 0;
+  a.baseMsgs = entries / a.runChannels;
+  a.extraChannels = entries % a.runChannels;
+  a.entriesBase = entries_for_msgs(a.baseMsgs, sh);
+  a.entriesExtra = entries_for_msgs(a.baseMsgs + 1, sh);
+  a.byParts = fast_div(static_cast<uint32_t>(a.parts));
+  a.byTeam = fast_div(static_cast<uint32_t>(a.team));
+  a.byCp = fast_div(static_cast<uint32_t>(a.cpSize));
+  a.byChannels = fast_div(static_cast<uint32_t>(a.runChannels));
+}
+
+hipError_t launch_exchange(const KernelArgs& args, int unitsPerPart, int maxParts, int teamUnits, hipStream_t stream) {
   KernelArgs a = args;
+  if (a.runChannels <= 0) return hipSuccess;
   const long runUnits = largest_run_units(a);
   const RunSplit split = split_for_run(runUnits, unitsPerPart, maxParts);
   a.parts = split.parts;
   a.unitsInFlight = split.unitsInFlight;
-  a.alignedStores = runUnits > static_cast<long>(kMaxUnitsInFlight) * kWaveLanes ? 1 : 0;
+  a.team = 1;
   int directions = (a.doSend ? 1 : 0) + (a.doRecv ? 1 : 0);
   int waves = directions * waves_per_direction(a) * a.parts;
   if (waves <= 0) return hipSuccess;
+  if (a.parts == 1 && teamUnits != 0) {
+    // Wavefronts that queue for slots anyway: a run of three or more passes goes to a team, one pass per
+    // wavefront (c4's three passes: -3 %; two passes, c5a: +2 %, so those stay with one wavefront).
+    const long perLane = (runUnits + kWaveLanes - 1) / kWaveLanes;
+    const long passes = (perLane + kMaxUnitsInFlight - 1) / kMaxUnitsInFlight;
+    if (teamUnits > 0 || (waves > kResidentWavefronts && passes >= 3)) {
+      const RunSplit team = split_for_run(runUnits, teamUnits > 0 ? teamUnits : kMaxUnitsInFlight, kMaxTeamWavefronts);
+      if (team.parts > 1) {
+        a.team = team.parts;
+        a.unitsInFlight = team.unitsInFlight;
+      }
+    }
+  }
+  a.alignedStores = runUnits > static_cast<long>(kMaxUnitsInFlight) * kWaveLanes ? 1 : 0;
+  set_launch_constants(a);
   if (a.parts > 1) {
     const int threads = directions * waves_per_direction(a);
     hipLaunchKernelGGL(helix_level_part_counters_kernel, dim3((threads + 255) / 256), dim3(256), 0, stream, a);
   }
-  // Wavefronts of a workgroup are independent (no LDS, no barrier). Two per workgroup dispatch and retire at
-  // the finest useful grain when wavefronts queue for slots; a launch that fits the device at once is bound
-  // by how fast its workgroups are dispatched, and four per workgroup halve that (c2: 7.2 -> 6.6 us).
-  const int wpb = waves <= kResidentWavefronts ? 4 : kWavesPerBlock;
-  int blocks = (waves + wpb - 1) / wpb;
+  // Wavefronts of a workgroup without teams are independent (no LDS, no barrier). Two per workgroup dispatch and
+  // retire at the finest useful grain when wavefronts queue for slots; a launch that fits the device at once is
+  // bound by how fast its workgroups are dispatched, and four per workgroup halve that (c2: 7.2 -> 6.6 us).
+  const int wpb = a.team > 1 ? a.team : waves <= kResidentWavefronts ? 4 : kWavesPerBlock;
+  int blocks = a.team > 1 ? waves : (waves + wpb - 1) / wpb;
+  a.wavesPerBlock = wpb;
   // Short runs: 1..6 units in flight, payload stored piece by piece. Long runs (more than one
   // pass of six; at least 4 units in flight by the rule): the instantiation whose receivers
   // realign the payload to 16-byte stores.
-#define HELIX_LAUNCH_EXCHANGE(K, ALIGNED) \
-  hipLaunchKernelGGL((helix_exchange_kernel<K, ALIGNED>), dim3(blocks), dim3(wpb * kWaveLanes), 0, stream, a)
+#define HELIX_LAUNCH_EXCHANGE(K, ALIGNED)                                                                                 \
+  do {                                                                                                                    \
+    if (a.team > 1)                                                                                                       \
+      hipLaunchKernelGGL((helix_exchange_kernel<K, ALIGNED, true>), dim3(blocks), dim3(wpb * kWaveLanes), 0, stream, a);  \
+    else                                                                                                                  \
+      hipLaunchKernelGGL((helix_exchange_kernel<K, ALIGNED, false>), dim3(blocks), dim3(wpb * kWaveLanes), 0, stream, a); \
+  } while (0)
   if (a.alignedStores && a.unitsInFlight >= 4) {
     switch (a.unitsInFlight) {
       case 4: HELIX_LAUNCH_EXCHANGE(4, true); break;
@@ -954,13 +1073,17 @@ hipError_t launch_exchange(const KernelArgs& args, int unitsPerPart, int maxPart
 
 hipError_t launch_combine(const KernelArgs& args, int parts, hipStream_t stream) {
   KernelArgs a = args;
-  a.parts = 1;  // the senders of this kernel walk whole runs
-  a.unitsInFlight = units_in_flight_for_run(largest_run_units(a));
-  const int senderStreams = a.doSend ? a.rankCount * a.runChannels * a.cpSize : 0;
   if (a.rankCount * a.runChannels <= 0) return hipSuccess;
   if (parts < 1) parts = 1;
   if (parts > kMaxCombineParts) parts = kMaxCombineParts;
-  const int blocks = (senderStreams + parts - 1) / parts + a.rankCount * a.runChannels;
+  a.parts = 1;  // the senders of this kernel walk whole runs
+  a.team = 1;
+  a.unitsInFlight = units_in_flight_for_run(largest_run_units(a));
+  set_launch_constants(a);
+  const int senderStreams = a.doSend ? a.rankCount * a.runChannels * a.cpSize : 0;
+  a.sendBlocks = (senderStreams + parts - 1) / parts;
+  a.wavesPerBlock = parts;
+  const int blocks = a.sendBlocks + a.rankCount * a.runChannels;
   dim3 block(static_cast<unsigned>(parts * kWaveLanes));
   // lanes per slot of the sideways pass: the smallest of 4, 8, 16, 32 that holds every sender
   const int g = a.cpSize <= 4 ? 4 : a.cpSize <= 8 ? 8 : a.cpSize <= 16 ? 16 : 32;

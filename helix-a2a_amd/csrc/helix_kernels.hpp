@@ -38,6 +38,15 @@ struct KernelArgs {
   int unitsInFlight;        // units_in_flight_for_run(largest run of the launch), 1..kMaxUnitsInFlight
   int alignedStores;        // receivers realign payload to 16-byte stores: set when runs take several passes
   int parts;                // wavefronts that share one stream's runs (per direction), 1..kMaxStreamParts
+  int team;                 // exchange kernel: wavefronts of a workgroup that walk one stream's run together (parts == 1), 1..kMaxTeamWavefronts
+  // Worked out by the launch functions from the fields above, so that no wavefront divides:
+  int np0, np;              // 8-byte pieces of field 0, of a message
+  int msgsPerEntry;         // messages one FIFO entry holds
+  int baseMsgs, extraChannels;  // channel c has baseMsgs + (c < extraChannels) messages in this launch
+  int entriesBase, entriesExtra;  // FIFO entries that baseMsgs and baseMsgs + 1 messages take
+  FastDiv byParts, byTeam, byCp, byChannels;
+  int sendBlocks;           // combine kernel: workgroups that send (the rest receive)
+  int wavesPerBlock;        // wavefronts of a workgroup of the launch
   uint64_t spinLimitTicks;  // bound of one in-kernel wait, in 100 MHz ticks
   uint32_t* status;         // device status word (HELIX_A2A_STATUS_* bits)
   // combine only
@@ -58,7 +67,12 @@ inline int waves_per_direction(const KernelArgs& a) { return a.rankCount * a.run
 
 // A stream's runs are shared by as many wavefronts (at most maxParts) as leave each at most
 // unitsPerPart units per lane; maxParts = 1: one wavefront per stream.
-hipError_t launch_exchange(const KernelArgs& a, int unitsPerPart, int maxParts, hipStream_t stream);
+// Teams (launches with one part per stream only): the wavefronts of a workgroup walk one stream's run together,
+// each a slice, sharing the stream's counters through the first of them. teamUnits -1: a launch whose wavefronts
+// queue for slots gives runs of three or more passes to teams, one pass per wavefront; 0: never; 1..6: always,
+// with at most that many units per lane and wavefront.
+constexpr int kMaxTeamWavefronts = 8;
+hipError_t launch_exchange(const KernelArgs& a, int unitsPerPart, int maxParts, int teamUnits, hipStream_t stream);
 // exchange fused with the LSE-weighted combine, all ranks of the launch; `parts` wavefronts share
 // the units of one (receiver, channel)
 constexpr int kMaxCombineParts = 8;

@@ -150,6 +150,32 @@ HELIX_HD uint32_t div_by_magic(uint32_t p, uint32_t magic) {
 #endif
 }
 
+// floor(n / d) for any n < 2^31 and 1 <= d < 2^31 without a divide and without a branch:
+// q = (mulhi(n, m) + n) >> s with s = ceil(log2 d) and m = floor(2^32 * (2^s - d) / d) + 1, that is a
+// multiplication by M = 2^32 + m = floor(2^(32+s) / d) + 1 (exact because 2^(32+s) < M*d <= 2^(32+s) + 2^s;
+// the sum cannot overflow for n < 2^31; d == 1 gives m = 1, s = 0, the identity). The host works the pair
+// out once per launch; wavefronts find their stream from their index with it.
+struct FastDiv {
+  uint32_t magic;
+  uint32_t shift;
+};
+HELIX_HD FastDiv fast_div(uint32_t d) {
+  FastDiv f;
+  if (d < 1u) d = 1u;
+  uint32_t s = 0;
+  while ((1ull << s) < d) ++s;
+  f.magic = static_cast<uint32_t>((((1ull << s) - d) << 32) / d) + 1u;
+  f.shift = s;
+  return f;
+}
+HELIX_HD uint32_t fast_div_by(uint32_t n, FastDiv f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return (__umulhi(n, f.magic) + n) >> f.shift;
+#else
+  return (static_cast<uint32_t>((static_cast<uint64_t>(n) * f.magic) >> 32) + n) >> f.shift;
+#endif
+}
+
 // Where unit U of a run lives: the message and the piece inside that message
 // of each of its two words. Unit U sits at byte U*16 of the FIFO entry.
 struct RunUnit {
@@ -258,15 +284,18 @@ HELIX_HD int auto_max_parts(int cpSize, int runChannels, int cuCount) {
 struct Slice {
   uint32_t begin, end;
 };
-HELIX_HD Slice slice_of_run(uint32_t runUnits, int part, int parts) {
+HELIX_HD Slice slice_of_run(uint32_t runUnits, int part, int parts, FastDiv byParts) {
   const uint32_t perLane = (runUnits + kWaveLanes - 1) / kWaveLanes;
-  const uint32_t slice = (perLane + parts - 1) / parts * kWaveLanes;
+  const uint32_t slice = fast_div_by(perLane + parts - 1, byParts) * kWaveLanes;
   Slice s;
   s.begin = static_cast<uint32_t>(part) * slice;
   if (s.begin > runUnits) s.begin = runUnits;
   s.end = s.begin + slice;
   if (s.end > runUnits) s.end = runUnits;
   return s;
+}
+HELIX_HD Slice slice_of_run(uint32_t runUnits, int part, int parts) {
+  return slice_of_run(runUnits, part, parts, fast_div(static_cast<uint32_t>(parts)));
 }
 
 }  // namespace helix

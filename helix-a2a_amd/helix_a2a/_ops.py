@@ -86,6 +86,8 @@ def _load_library() -> ctypes.CDLL:
     lib.helix_a2a_alltoall_loopback_static.restype = ctypes.c_int
     lib.helix_a2a_set_units_per_wavefront.argtypes = [ctypes.c_int]
     lib.helix_a2a_set_units_per_wavefront.restype = ctypes.c_int
+    lib.helix_a2a_set_team_units.argtypes = [ctypes.c_int]
+    lib.helix_a2a_set_team_units.restype = ctypes.c_int
     lib.helix_a2a_alltoall_combine_loopback.argtypes = [
         P(_Params), P(_CombineOut), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
     lib.helix_a2a_alltoall_combine_loopback.restype = ctypes.c_int
@@ -783,6 +785,11 @@ def set_spin_limit_us(microseconds: int) -> None:
 def set_units_per_wavefront(units: int) -> None:
     """Share a stream's runs longer than ``units`` KiB between wavefronts: 1..6 always, 0 never, -1 (default) beyond 6 KiB while the launch leaves the device under-filled."""
     _check(_lib.helix_a2a_set_units_per_wavefront(int(units)), "set_units_per_wavefront")
+
+
+def set_team_units(units: int) -> None:
+    """Let the wavefronts of a workgroup walk one stream's run together: 1..6 always (units per lane and wavefront), 0 never, -1 (default) runs of three or more passes in launches whose wavefronts queue."""
+    _check(_lib.helix_a2a_set_team_units(int(units)), "set_team_units")
 
 
 def set_checked_mode(enabled: bool) -> None:

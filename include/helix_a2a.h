@@ -286,6 +286,24 @@ void helix_a2a_set_single_round(int enabled);
  */
 int helix_a2a_set_units_per_wavefront(int units);
 
+/*
+ * Teams (process-wide; takes effect with the next call). In a launch that
+ * keeps one wavefront per stream and direction, the wavefronts of a workgroup
+ * can walk one stream's run together, each a slice of it: only the first of
+ * them touches the stream's counters and hands the step to the others through
+ * LDS, so the same bytes move in more, shorter wavefronts without any more
+ * counter traffic, and the two halves of an exchange may differ in it.
+ *   -1 (default)  runs of three or more passes (more than 12 units per lane)
+ *                 in a launch whose wavefronts queue for slots: one pass per
+ *                 wavefront, at most 8 wavefronts
+ *    0            never
+ *    1..6         always, with at most that many units per lane and wavefront
+ * No counterpart in the reference, which keeps one warp per stream whatever
+ * its length (csrc/helix_alltoall.cu:315-334). Returns 0 or
+ * HELIX_A2A_ERR_INVALID_ARGUMENT.
+ */
+int helix_a2a_set_team_units(int units);
+
 /* thread-local message of the most recent failure on this thread ("" if none) */
 const char* helix_a2a_last_error(void);
 

@@ -85,6 +85,10 @@ class HostModel:
         lib.hm_div.restype = ctypes.c_uint32
         lib.hm_div_mismatches.argtypes = [ctypes.c_uint32]
         lib.hm_div_mismatches.restype = ctypes.c_int
+        lib.hm_fast_div.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
+        lib.hm_fast_div.restype = ctypes.c_uint32
+        lib.hm_fast_div_mismatches.argtypes = [ctypes.c_uint32, ctypes.c_int]
+        lib.hm_fast_div_mismatches.restype = ctypes.c_int
         lib.hm_run_lines.argtypes = [ctypes.c_int] * 3
         lib.hm_run_lines.restype = ctypes.c_int
         lib.hm_msgs_per_entry.argtypes = [ctypes.c_int] * 2

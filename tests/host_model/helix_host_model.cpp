@@ -354,6 +354,36 @@ int hm_div_mismatches(uint32_t d) {
     bad += div_by_magic(g, magic) != g / d;
   return bad;
 }
+// floor(n / d) the way wavefronts find their stream from their index (any n < 2^31)
+uint32_t hm_fast_div(uint32_t n, uint32_t d) { return fast_div_by(n, fast_div(d)); }
+// number of n among multiples of d, their neighbours, small values, 2^31 - 1 and `samples` pseudo-random values for
+// which that differs from n / d
+int hm_fast_div_mismatches(uint32_t d, int samples) {
+  int bad = 0;
+  const FastDiv f = fast_div(d);
+  auto check = [&](uint64_t n) {
+    if (n < (1ull << 31)) bad += fast_div_by(static_cast<uint32_t>(n), f) != static_cast<uint32_t>(n) / d;
+  };
+  for (uint64_t n = 0; n < 300; ++n) check(n);
+  for (uint64_t k = 1; k < 300; ++k) {
+    check(k * d - 1);
+    check(k * d);
+    check(k * d + 1);
+  }
+  const uint64_t top = ((1ull << 31) - 1) / d * d;
+  check(top - 1);
+  check(top);
+  check(top + 1);
+  check((1ull << 31) - 1);
+  uint64_t x = 88172645463325252ull + d;
+  for (int i = 0; i < samples; ++i) {
+    x ^= x << 13;
+    x ^= x >> 7;
+    x ^= x << 17;
+    check(x & 0x7fffffffull);
+  }
+  return bad;
+}
 // lines of a run of `msgs` messages and messages per FIFO entry for a message of the two field sizes
 int hm_run_lines(int msgs, int field0_bytes, int field1_bytes) { return run_lines(msgs, make_msg_shape(field0_bytes, field1_bytes)); }
 int hm_msgs_per_entry(int field0_bytes, int field1_bytes) { return msgs_per_fifo_entry(make_msg_shape(field0_bytes, field1_bytes)); }

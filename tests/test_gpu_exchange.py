@@ -580,6 +580,68 @@ def test_fifo_image_matches_host_model(hx, ops, host_model):
 # bounded waits and back-pressure
 # ---------------------------------------------------------------------------
 
+@pytest.mark.parametrize("units", [1, 2, 3, 5, 6])
+def test_runs_walked_by_teams(hx, ops, units):
+    # the wavefronts of a workgroup walk one stream's run together (slices of at most `units` units per lane),
+    # sharing its counters through the first of them: same bits as one wavefront per stream, call after call
+    # on one workspace, for runs of one and of many passes, several runs per launch, ragged message sizes
+    shapes = [(3, 7, 1096, 6, 2), (8, 256, 1024, 16, 128), (2, 9, 61432, 2, 1), (4, 12, 1016, 14, 1), (16, 64, 264, 2, 4),
+              (2, 400, 8, 6, 2), (5, 26, 600, 2, 2)]
+    try:
+        ops.set_units_per_wavefront(0)  # one part per stream: the launches teams apply to
+        for cp, entries, x, s, channels in shapes:
+            ws = get_workspace(hx, cp)
+            g = torch.Generator().manual_seed(cp * 37 + entries + units)
+            ins_o = [torch.randint(-32768, 32767, (entries, cp, x), generator=g, dtype=torch.int16).view(torch.bfloat16).cuda()
+                     for _ in range(cp)]
+            ins_s = [torch.randint(-2**31, 2**31 - 1, (entries, cp, s), generator=g, dtype=torch.int32).view(torch.float32).cuda()
+                     for _ in range(cp)]
+            for u in (units, 0, units):
+                ops.set_team_units(u)
+                outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws, channel_count=channels)
+                torch.cuda.synchronize()
+                assert_clean(ops)
+                check_against_oracle(ins_o, ins_s, outs_o, outs_s, with_numpy=False)
+    finally:
+        ops.set_team_units(-1)
+        ops.set_units_per_wavefront(-1)
+    with pytest.raises(RuntimeError, match="units per team wavefront"):
+        ops.set_team_units(7)
+
+
+def test_team_whose_wait_gives_up_leaves_together(hx, ops):
+    # receivers without senders, as teams: the first wavefront of each team gives up its wait and every
+    # wavefront of the team leaves with it; the kernel ends normally and reports the time-out
+    cp = 2
+    ws = get_workspace(hx, cp, fresh=True)
+    o = [torch.zeros(3, cp, 2048, dtype=torch.bfloat16, device="cuda") for _ in range(cp)]
+    s = [torch.zeros(3, cp, 2, device="cuda") for _ in range(cp)]
+    out_o = [torch.empty_like(t) for t in o]
+    out_s = [torch.empty_like(t) for t in s]
+    arr = (ops._Params * cp)()
+    for r in range(cp):
+        arr[r] = ops._make_params(o[r], s[r], out_o[r], out_s[r], ws, r, cp, 1)
+    ops.set_spin_limit_us(0)  # every wait gives up at its first clock check
+    ops.set_units_per_wavefront(0)
+    ops.set_team_units(2)
+    try:
+        ops._check(ops._lib.helix_a2a_alltoall_recv(arr, cp, ops._stream_handle()), "recv")
+        torch.cuda.synchronize()
+        status = ops.device_status()
+    finally:
+        ops.set_spin_limit_us(2_000_000)
+        ops.set_team_units(-1)
+        ops.set_units_per_wavefront(-1)
+    assert status & 1, "the receiving teams should have reported a timed-out wait"
+    for r in range(cp):
+        hx.init_workspace(ws, r, cp)
+    ins_o = [torch.randn(3, cp, 2048, device="cuda").to(torch.bfloat16) for _ in range(cp)]
+    outs_o, outs_s = hx.alltoall_loopback(ins_o, s, ws, channel_count=1)
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(ins_o, s, outs_o, outs_s, with_numpy=False)
+
+
 def test_receive_without_send_times_out_cleanly(hx, ops):
     cp = 2
     ws = get_workspace(hx, cp, fresh=True)

@@ -218,6 +218,16 @@ def test_receiver_rejects_stale_lines(host_model):
     assert rc > 0 and "flag" in msg
 
 
+def test_stream_of_a_wavefront_without_a_divide(host_model):
+    # wavefronts find (part, peer, channel, rank) from their index with a multiply-high, an add and a shift per
+    # divisor; exact for every index below 2^31 and every divisor a launch can have (parts, cp, channels)
+    lib = host_model.lib
+    for d in list(range(1, 4100)) + [4999, 65535, 65536, 65537, 10**6 + 3, 2**20, 2**24 - 1, 2**30, 2**30 + 1, 2**31 - 1]:
+        assert lib.hm_fast_div_mismatches(d, 200) == 0, d
+    assert [lib.hm_fast_div(n, 7) for n in (0, 6, 7, 13, 14, 2**31 - 1)] == [0, 0, 1, 1, 2, (2**31 - 1) // 7]
+    assert lib.hm_fast_div(12345, 1) == 12345
+
+
 def test_split_rule(host_model):
     # wavefronts per stream: as many as leave each at most `units per part` units per lane (16 at most);
     # units in flight: the slice of a part in the fewest passes of at most 6, then the smallest such count
