@@ -2,16 +2,26 @@
 //
 // One wavefront owns one stream = (sender rank, receiver rank, channel) in one
 // direction, the role a warp has in the reference kernel
-// (csrc/helix_alltoall.cu:315-474); a long run in a launch that leaves the device
-// under-filled is shared by several wavefronts, each with a slice of its own.
+// (csrc/helix_alltoall.cu:315-474). A long run is shared by several wavefronts,
+// each with a slice of its own: wavefronts with counters of their own ("parts")
+// in a launch that leaves the device under-filled, the wavefronts of one
+// workgroup behind one set of counters (a "team") in a launch that fills it.
 // A sender wavefront reads its messages from the send tensors, turns them into
 // LL128 lines in registers, stores the lines into the receiver's FIFO and, once
 // those stores are acknowledged, moves its step counter: that is the token its
 // receiver waits for. A receiver wavefront then reads the lines in one pass,
 // checks that their flags carry the step, and stores the payload into the
-// receive tensors. There is no staging copy and no barrier: data moves
+// receive tensors. There is no staging copy: data moves
 // global -> registers -> FIFO -> registers -> global, 16 bytes per lane on
-// the FIFO side.
+// the FIFO side. Nothing but a team's step goes through LDS, and only teams
+// meet at a barrier.
+//
+// No wavefront divides: what follows from the shape of a launch (pieces per
+// message, messages per channel, the divisors that turn a wavefront's index
+// into its stream) is worked out by the host and travels in the argument
+// block, which every wavefront fetches with a few wide scalar loads at its
+// very start. Before that, a wavefront spent a dozen dependent trips to the
+// scalar cache and six software divisions ahead of its first payload load.
 //
 // Why the token and not the flags alone: a 64-lane 16-byte load of eight lines
 // is served in 64-byte halves, and the flag word of a line sits in its second

@@ -57,7 +57,7 @@ struct KernelArgs {
   uint32_t np0Magic;   // div_magic(pieces of field 0)
 };
 
-// Wavefronts of a workgroup of the exchange kernel are independent (no LDS, no barrier); small
+// Wavefronts of a workgroup of the exchange kernel are independent unless they form a team (no LDS, no barrier); small
 // workgroups dispatch and retire at a finer grain (2 measured best of 1..16 on launches that queue).
 constexpr int kWavesPerBlock = 2;
 constexpr int kResidentWavefronts = 4096;  // 256 CUs x 4 SIMDs x 4 wavefronts: what runs at once
