@@ -508,7 +508,7 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
       }
       if (__ballot(!flagsAgree) != 0ull) {
         raise_status(a, kStatusInternal, lane);
-        return;
+        if (!kTeam) return;  // a wavefront of a team stays with its team to the last barrier; the workspace is marked broken
       }
       if (U0 == slice.begin && firstMsg == 0) HELIX_MARK(wave, 1, false);
 #pragma unroll

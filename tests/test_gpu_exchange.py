@@ -642,6 +642,52 @@ def test_team_whose_wait_gives_up_leaves_together(hx, ops):
     check_against_oracle(ins_o, s, outs_o, outs_s, with_numpy=False)
 
 
+@pytest.mark.parametrize("teams", [False, True])
+def test_corrupt_line_is_reported(hx, ops, teams):
+    # a line whose flag word does not carry the step once the token says the run is complete: the receiver
+    # reports a corrupt workspace (status bit 4), the kernel ends normally, and the workspace stays out of use
+    # (bit 8) until it is initialised again -- for single wavefronts and for teams alike
+    cp, entries, channels = 2, 3, 1
+    ws = get_workspace(hx, cp, fresh=True)
+    g = torch.Generator().manual_seed(5)
+    o = [torch.randint(-32768, 32767, (entries, cp, 2048), generator=g, dtype=torch.int16).view(torch.bfloat16).cuda()
+         for _ in range(cp)]
+    s = [torch.zeros(entries, cp, 2, device="cuda") for _ in range(cp)]
+    out_o = [torch.zeros_like(t) for t in o]
+    out_s = [torch.zeros_like(t) for t in s]
+    arr = (ops._Params * cp)()
+    for r in range(cp):
+        arr[r] = ops._make_params(o[r], s[r], out_o[r], out_s[r], ws, r, cp, channels)
+    try:
+        if teams:
+            ops.set_units_per_wavefront(0)
+            ops.set_team_units(2)
+        ops._check(ops._lib.helix_a2a_alltoall_send(arr, cp, ops._stream_handle()), "send")
+        torch.cuda.synchronize()
+        assert ops.device_status() == 0
+        # the FIFO of stream (sender 0 -> receiver 1, channel 0) starts receiver 1's row; a fresh workspace is at
+        # step 0, entry 0; the flag word is the last 8 bytes of a 128-byte line
+        line = 37
+        assert int(ws[1, line * 16 + 15]) == 0, "the flag word of a line of step 0"
+        ws[1, line * 16 + 15] = 12345
+        ops._check(ops._lib.helix_a2a_alltoall_recv(arr, cp, ops._stream_handle()), "recv")
+        torch.cuda.synchronize()
+        status = ops.device_status()
+        assert status & ops.STATUS_INTERNAL, status
+        hx.alltoall_loopback(o, s, ws, channel_count=channels)
+        torch.cuda.synchronize()
+        assert ops.device_status() & ops.STATUS_BROKEN_WORKSPACE
+    finally:
+        ops.set_team_units(-1)
+        ops.set_units_per_wavefront(-1)
+        for r in range(cp):
+            hx.init_workspace(ws, r, cp)
+    outs_o, outs_s = hx.alltoall_loopback(o, s, ws, channel_count=channels)
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(o, s, outs_o, outs_s, with_numpy=False)
+
+
 def test_receive_without_send_times_out_cleanly(hx, ops):
     cp = 2
     ws = get_workspace(hx, cp, fresh=True)
