@@ -39,12 +39,12 @@ PEAK_HBM_GBPS = 8000.0
 # <kernel>_<workload>.md hold the runs these come from. These counters sit between L2 and fabric:
 # they do not tell whether the memory-side cache or DRAM served a request.
 MEASURED_TRAFFIC_BYTES = {
-    ("helix_exchange_kernel", "c3", 128): 150_939_853,   # profiles/helix_exchange_kernel_c3.md
-    ("helix_exchange_kernel", "c4", 128): 566_596_958,   # profiles/helix_exchange_kernel_c4.md
-    ("helix_exchange_kernel", "c5a", 64): 600_281_026,   # profiles/helix_exchange_kernel_c5a.md
-    ("helix_combine_kernel", "c3", 128): 118_823_140,    # profiles/helix_combine_kernel_c3.md
-    ("helix_combine_kernel", "c4", 128): 451_944_228,    # profiles/helix_combine_kernel_c4.md
-    ("helix_combine_kernel", "c5a", 64): 464_338_670,    # profiles/helix_combine_kernel_c5a.md
+    ("helix_exchange_kernel", "c3", 128): 151_031_722,   # profiles/helix_exchange_kernel_c3.md
+    ("helix_exchange_kernel", "c4", 128): 566_613_588,   # profiles/helix_exchange_kernel_c4.md
+    ("helix_exchange_kernel", "c5a", 64): 587_707_467,   # profiles/helix_exchange_kernel_c5a.md
+    ("helix_combine_kernel", "c3", 128): 118_789_868,    # profiles/helix_combine_kernel_c3.md
+    ("helix_combine_kernel", "c4", 128): 451_874_147,    # profiles/helix_combine_kernel_c4.md
+    ("helix_combine_kernel", "c5a", 64): 464_327_337,    # profiles/helix_combine_kernel_c5a.md
 }
 
 

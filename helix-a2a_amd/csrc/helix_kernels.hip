@@ -205,7 +205,7 @@ __device__ __forceinline__ void fetch_scalars_up_front(const KernelArgs& a) {
                "s"(a.recvBytes1), "s"(a.npMagic), "s"(a.rankBegin), "s"(a.rankCount), "s"(a.doSend), "s"(a.doRecv));
   asm volatile("" ::"s"(a.parts), "s"(a.team), "s"(a.np0), "s"(a.np), "s"(a.msgsPerEntry), "s"(a.baseMsgs),
                "s"(a.extraChannels), "s"(a.byParts.magic), "s"(a.byParts.shift), "s"(a.byTeam.magic), "s"(a.byTeam.shift),
-               "s"(a.byCp.magic), "s"(a.byCp.shift), "s"(a.byChannels.magic), "s"(a.byChannels.shift), "s"(a.sendBlocks), "s"(a.wavesPerBlock),
+               "s"(a.byCp.magic), "s"(a.byCp.shift), "s"(a.byChannels.magic), "s"(a.byChannels.shift), "s"(a.sendBlocks), "s"(a.wavesPerBlock), "s"(a.dirBlocks), "s"(a.xcdGroup),
                "s"(a.spinLimitTicks));
 }
 
@@ -607,13 +607,13 @@ __global__ __launch_bounds__(1024) HELIX_WAVES_PER_SIMD void helix_exchange_kern
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWaveLanes);
   const int lane = static_cast<int>(threadIdx.x) % kWaveLanes;
   const int probe = static_cast<int>(blockIdx.x) * a.wavesPerBlock + wave;  // index of the wavefront in the launch
-  int w = kTeam ? static_cast<int>(blockIdx.x) : probe;
+  // Workgroups of the sending direction come first, a.dirBlocks of them, then as many that receive.
+  const bool isSender = a.doSend != 0 && static_cast<int>(blockIdx.x) < a.dirBlocks;
+  int block = static_cast<int>(blockIdx.x) - (a.doSend != 0 && !isSender ? a.dirBlocks : 0);
+  block = xcd_grouped(block, a.xcdGroup);
+  const int w = kTeam ? block : block * a.wavesPerBlock + wave;
   const int perDirection = a.rankCount * a.runChannels * a.cpSize * a.parts;
-  const int senders = a.doSend ? perDirection : 0;
-  const int total = senders + (a.doRecv ? perDirection : 0);
-  if (w >= total) return;
-  const bool isSender = w < senders;
-  if (!isSender) w -= senders;
+  if (w >= perDirection) return;
   const int q = static_cast<int>(fast_div_by(static_cast<uint32_t>(w), a.byParts));
   const int part = kTeam ? wave : w - q * a.parts;
   const int t = static_cast<int>(fast_div_by(static_cast<uint32_t>(q), a.byCp));
@@ -998,6 +998,18 @@ static long largest_run_units(const KernelArgs& a) {
   return run_units(msgs < perEntry ? msgs : perEntry, sh);
 }
 
+// The `group` of xcd_grouped for a launch direction of `blocks` workgroups of `wavesPerBlock` wavefronts in which
+// `wavesPerPeerSet` consecutive wavefronts serve the peers of one (rank, channel), `streamsPerBlock` of them to
+// a workgroup: the workgroups of one peer set, if the statistics rows of different workgroups share 128-byte
+// lines at all and the tiling fits; else 0 (as dispatched). A power of two.
+static int xcd_group_for(int wavesPerPeerSet, int wavesPerBlock, int streamsPerBlock, int blocks, int field1Bytes) {
+  if (field1Bytes * streamsPerBlock >= 128) return 0;  // the rows a workgroup touches fill whole lines
+  if (wavesPerPeerSet % wavesPerBlock != 0) return 0;
+  const int group = wavesPerPeerSet / wavesPerBlock;
+  if (group < 2 || (group & (group - 1)) != 0 || blocks % (8 * group) != 0) return 0;
+  return group;
+}
+
 // The fields of the argument block that follow from the others (see KernelArgs); a.parts and a.team are set.
 static void set_launch_constants(KernelArgs& a) {
   const MsgShape sh = make_msg_shape(a.field0Bytes, a.field1Bytes);
@@ -1049,7 +1061,11 @@ hipError_t launch_exchange(const KernelArgs& args, int unitsPerPart, int maxPart
   // retire at the finest useful grain when wavefronts queue for slots; a launch that fits the device at once is
   // bound by how fast its workgroups are dispatched, and four per workgroup halve that (c2: 7.2 -> 6.6 us).
   const int wpb = a.team > 1 ? a.team : waves <= kResidentWavefronts ? 4 : kWavesPerBlock;
-  int blocks = a.team > 1 ? waves : (waves + wpb - 1) / wpb;
+  const int perDirection = waves / directions;
+  a.dirBlocks = a.team > 1 ? perDirection : (perDirection + wpb - 1) / wpb;
+  // (launches with teams stay as dispatched: regrouped, c4 in the per-head layout took 0.7 % longer)
+  a.xcdGroup = a.team > 1 ? 0 : xcd_group_for(a.cpSize * a.parts, wpb, a.parts > 1 ? 1 : wpb, a.dirBlocks, a.field1Bytes);
+  int blocks = directions * a.dirBlocks;
   a.wavesPerBlock = wpb;
   // Short runs: 1..6 units in flight, payload stored piece by piece. Long runs (more than one
   // pass of six; at least 4 units in flight by the rule): the instantiation whose receivers
@@ -1093,6 +1109,8 @@ hipError_t launch_combine(const KernelArgs& args, int parts, hipStream_t stream)
   const int senderStreams = a.doSend ? a.rankCount * a.runChannels * a.cpSize : 0;
   a.sendBlocks = (senderStreams + parts - 1) / parts;
   a.wavesPerBlock = parts;
+  a.dirBlocks = a.sendBlocks;
+  a.xcdGroup = 0;  // regrouping the sending workgroups of this kernel was measured: nothing at c3 / c5a, +1.3 % at c4
   const int blocks = a.sendBlocks + a.rankCount * a.runChannels;
   dim3 block(static_cast<unsigned>(parts * kWaveLanes));
   // lanes per slot of the sideways pass: the smallest of 4, 8, 16, 32 that holds every sender

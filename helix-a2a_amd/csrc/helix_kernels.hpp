@@ -47,6 +47,8 @@ struct KernelArgs {
   FastDiv byParts, byTeam, byCp, byChannels;
   int sendBlocks;           // combine kernel: workgroups that send (the rest receive)
   int wavesPerBlock;        // wavefronts of a workgroup of the launch
+  int dirBlocks;            // workgroups per direction (combine kernel: that send)
+  int xcdGroup;             // consecutive workgroups' worth of streams that one XCD serves (xcd_grouped), 0: as dispatched
   uint64_t spinLimitTicks;  // bound of one in-kernel wait, in 100 MHz ticks
   uint32_t* status;         // device status word (HELIX_A2A_STATUS_* bits)
   // combine only

@@ -85,6 +85,8 @@ class HostModel:
         lib.hm_div.restype = ctypes.c_uint32
         lib.hm_div_mismatches.argtypes = [ctypes.c_uint32]
         lib.hm_div_mismatches.restype = ctypes.c_int
+        lib.hm_xcd_grouped.argtypes = [ctypes.c_int, ctypes.c_int]
+        lib.hm_xcd_grouped.restype = ctypes.c_int
         lib.hm_fast_div.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
         lib.hm_fast_div.restype = ctypes.c_uint32
         lib.hm_fast_div_mismatches.argtypes = [ctypes.c_uint32, ctypes.c_int]

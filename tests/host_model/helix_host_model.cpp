@@ -354,6 +354,8 @@ int hm_div_mismatches(uint32_t d) {
     bad += div_by_magic(g, magic) != g / d;
   return bad;
 }
+// the place workgroup `block` takes when `group` consecutive workgroups' worth of streams go to one XCD
+int hm_xcd_grouped(int block, int group) { return xcd_grouped(block, group); }
 // floor(n / d) the way wavefronts find their stream from their index (any n < 2^31)
 uint32_t hm_fast_div(uint32_t n, uint32_t d) { return fast_div_by(n, fast_div(d)); }
 // number of n among multiples of d, their neighbours, small values, 2^31 - 1 and `samples` pseudo-random values for

@@ -228,6 +228,23 @@ def test_stream_of_a_wavefront_without_a_divide(host_model):
     assert lib.hm_fast_div(12345, 1) == 12345
 
 
+def test_workgroups_regrouped_by_xcd(host_model):
+    # workgroup i runs on XCD i mod 8; within tiles of 8 * group workgroups the regrouping is a permutation that
+    # gives every XCD `group` consecutive places, and it leaves a launch alone when group is 0
+    f = host_model.lib.hm_xcd_grouped
+    for group in (2, 4, 8, 16):
+        tile = 8 * group
+        n = 5 * tile
+        places = [f(b, group) for b in range(n)]
+        assert sorted(places) == list(range(n))
+        for t in range(0, n, tile):
+            assert sorted(places[t:t + tile]) == list(range(t, t + tile))      # a tile stays a tile
+            for xcd in range(8):
+                mine = sorted(places[b] for b in range(t, t + tile) if b % 8 == xcd)
+                assert mine == list(range(t + xcd * group, t + (xcd + 1) * group))  # consecutive places per XCD
+    assert [f(b, 0) for b in range(20)] == list(range(20))
+
+
 def test_split_rule(host_model):
     # wavefronts per stream: as many as leave each at most `units per part` units per lane (16 at most);
     # units in flight: the slice of a part in the fewest passes of at most 6, then the smallest such count
