@@ -561,7 +561,7 @@ int helix_a2a_alltoall_combine_loopback(const helix_a2a_params_t* per_rank, cons
     int msgs = stream_msg_count(a.entryBegin, a.entryEnd, 0, a.runChannels);
     int perEntry = msgs_per_fifo_entry(plan.shape);
     long runPieces = static_cast<long>(msgs < perEntry ? msgs : perEntry) * plan.shape.np0;
-    long perTurn = (cp_size <= 8 ? 2 : 1) * kWaveLanes;  // pieces a wavefront takes per turn
+    long perTurn = (cp_size <= 16 ? 2 : 1) * kWaveLanes;  // pieces a wavefront takes per turn
     long cover = (runPieces + perTurn - 1) / perTurn;
     long fill = static_cast<long>(plan.cuCount) * 16 / (static_cast<long>(cp_size) * a.runChannels);
     long parts = cover < fill ? cover : fill;

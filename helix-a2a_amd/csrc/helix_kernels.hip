@@ -665,8 +665,9 @@ __device__ __forceinline__ void widen4<1>(u32x2 piece, float (&f)[4]) {  // fp16
 // wavefront turns sideways -- lane i serves slot i / G and sender i % G, loads that sender's
 // statistics of that head, and a softmax over the G lanes of a slot gives the weight -- and the
 // weights go back through LDS to the lanes that own pieces of the head. (G = 4, 8, 16 or 32 lanes
-// per slot for cpSize <= 4, 8, 16, 32.) With up to eight senders a lane handles two accesses per
-// turn, so that sixteen loads are in flight either way.
+// per slot for cpSize <= 4, 8, 16, 32.) With up to sixteen senders a lane handles two accesses per
+// turn (sixteen loads in flight with eight senders, thirty-two with sixteen: c5a -1 % against one
+// access), with more senders one.
 constexpr int kCombineSlots = 32;  // distinct (message, head) pairs one turn may touch (head_dim >= 32: at most 18)
 
 struct CombineCtx {
@@ -741,7 +742,7 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
                                                      int lane, CombineLds<kLanesPerSlot>& lds, int probe) {
   HELIX_MARK(probe, 0, false);
   constexpr int kSlotsPerPass = kWaveLanes / kLanesPerSlot;
-  constexpr int kAccesses = kLanesPerSlot <= 8 ? 2 : 1;                  // accesses a lane handles per turn
+  constexpr int kAccesses = kLanesPerSlot <= 16 ? 2 : 1;                  // accesses a lane handles per turn
   constexpr int kGroup = kLanesPerSlot <= 16 ? kLanesPerSlot : 16;       // senders whose pieces are in flight together
   Stream st;
   setup_stream(st, a, 0, ch);
