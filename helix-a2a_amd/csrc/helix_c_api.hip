@@ -378,6 +378,9 @@ int read_status(DeviceState* st, hipStream_t stream, uint32_t* out) {
 // End of every exchange call: nothing in the normal mode, a synchronous status check in checked mode.
 int finish_call(int rc, hipStream_t stream) {
   if (rc != HELIX_A2A_OK || !checked_mode()) return rc;
+  // a stream that is being captured into a graph cannot be waited for: the check is left to the replays' caller
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone) return rc;
   DeviceState* st = nullptr;
   if ((rc = device_state(&st))) return rc;
   uint32_t status = 0;

@@ -247,8 +247,9 @@ int helix_a2a_device_status(uint32_t* status, void* stream);
  * helix_a2a_set_checked_mode(1): every exchange call waits for its stream and
  * reads the status word before it returns, and returns HELIX_A2A_ERR_DEVICE
  * (message: the bits) if it is not zero. For bring-up and tests; it makes the
- * calls synchronous. Default 0. The environment variable HELIX_A2A_CHECKED=1
- * switches it on from the start.
+ * calls synchronous. A call on a stream that is being captured into a graph
+ * cannot wait and skips the check. Default 0. The environment variable
+ * HELIX_A2A_CHECKED=1 switches it on from the start.
  */
 void helix_a2a_set_checked_mode(int enabled);
 

@@ -33,6 +33,16 @@ def ops(hx):
 _WORKSPACES = {}
 
 
+@pytest.fixture
+def unchecked(ops):
+    """For tests that make a kernel fail on purpose and read the status word themselves: checked mode off,
+    whatever HELIX_A2A_CHECKED says, and back to what it says afterwards."""
+    import os
+    ops.set_checked_mode(False)
+    yield
+    ops.set_checked_mode(os.environ.get("HELIX_A2A_CHECKED", "") not in ("", "0"))
+
+
 def get_workspace(hx, cp, fresh=False):
     """One workspace per cp for the whole module (4.3 GB at cp = 8), initialised on first use."""
     ws = _WORKSPACES.get(cp)
@@ -609,7 +619,7 @@ def test_runs_walked_by_teams(hx, ops, units):
         ops.set_team_units(7)
 
 
-def test_team_whose_wait_gives_up_leaves_together(hx, ops):
+def test_team_whose_wait_gives_up_leaves_together(hx, ops, unchecked):
     # receivers without senders, as teams: the first wavefront of each team gives up its wait and every
     # wavefront of the team leaves with it; the kernel ends normally and reports the time-out
     cp = 2
@@ -643,7 +653,7 @@ def test_team_whose_wait_gives_up_leaves_together(hx, ops):
 
 
 @pytest.mark.parametrize("teams", [False, True])
-def test_corrupt_line_is_reported(hx, ops, teams):
+def test_corrupt_line_is_reported(hx, ops, teams, unchecked):
     # a line whose flag word does not carry the step once the token says the run is complete: the receiver
     # reports a corrupt workspace (status bit 4), the kernel ends normally, and the workspace stays out of use
     # (bit 8) until it is initialised again -- for single wavefronts and for teams alike
@@ -688,7 +698,7 @@ def test_corrupt_line_is_reported(hx, ops, teams):
     check_against_oracle(o, s, outs_o, outs_s, with_numpy=False)
 
 
-def test_receive_without_send_times_out_cleanly(hx, ops):
+def test_receive_without_send_times_out_cleanly(hx, ops, unchecked):
     cp = 2
     ws = get_workspace(hx, cp, fresh=True)
     o = [torch.zeros(3, cp, 64, dtype=torch.bfloat16, device="cuda") for _ in range(cp)]
@@ -711,7 +721,7 @@ def test_receive_without_send_times_out_cleanly(hx, ops):
         hx.init_workspace(ws, r, cp)
 
 
-def test_exchange_after_a_timeout_does_nothing_until_reinit(hx, ops):
+def test_exchange_after_a_timeout_does_nothing_until_reinit(hx, ops, unchecked):
     # a wait that gives up marks the workspace broken: the exchanges queued behind it write nothing and say so
     cp = 4
     ws = get_workspace(hx, cp, fresh=True)
@@ -958,7 +968,7 @@ def test_exchange_and_combine_replay_from_a_captured_graph(hx, ops):
 # helix_a2a_alltoall: both halves of one rank in one launch (what one process per GPU would call)
 # ---------------------------------------------------------------------------
 
-def test_single_rank_call_both_halves(hx, ops):
+def test_single_rank_call_both_halves(hx, ops, unchecked):
     import ctypes
 
     # cp_size 1: the rank is its own peer, the launch sends and receives its own traffic
