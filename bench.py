@@ -249,6 +249,9 @@ def main() -> int:
                          "that must not mix launches of the two legs")
     ap.add_argument("--units-per-wavefront", type=int, default=None, metavar="U",
                     help="share runs longer than U KiB per wavefront between wavefronts (library default: 6; 0 = never)")
+    ap.add_argument("--team-units", type=int, default=None, metavar="U",
+                    help="teams of wavefronts per stream: 1..6 always (at most U KiB per wavefront), 0 never, "
+                         "-1 the library's rule (runs of three or more passes in launches that queue)")
     ap.add_argument("--no-host-timing", action="store_true", help="skip the host-time-per-call measurements")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
@@ -277,6 +280,8 @@ def main() -> int:
         helix_a2a.init_workspace(ws, r, w.cp)
     if args.units_per_wavefront is not None:
         _ops.set_units_per_wavefront(args.units_per_wavefront)
+    if args.team_units is not None:
+        _ops.set_team_units(args.team_units)
     ins_o, ins_s = make_inputs(w, "cuda")
     entries = w.tokens
     if args.layout == "head":
