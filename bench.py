@@ -32,6 +32,7 @@ for _p in (ROOT / "helix-a2a_amd", ROOT):
 
 METRIC = "µs/call + effective HBM GB/s (% of peak) for Helix a2a, cp=4/8, 1 GPU"
 PEAK_HBM_GBPS = 8000.0
+MIN_ROOFLINE_STEPS = 200
 
 # Bytes that crossed between the L2s and the fabric per launch (FETCH_SIZE + WRITE_SIZE of two
 # rocprofv3 --pmc runs, each scaled by the same counter of a plain copy kernel), one row per profiled
@@ -59,7 +60,7 @@ def cpu_baseline(w, algorithmic_bytes: int, budget_s: float = 12.0):
     """Time the CPU restatements on this host for the same workload (bounded sample)."""
     import torch
 
-    from helix_a2a.workloads import make_inputs
+    from helix_workloads import make_inputs
     from oracle import helix_oracle as ho
 
     ins_o, ins_s = make_inputs(w, "cpu")
@@ -130,7 +131,6 @@ def host_timing(w, ws, ins_o, ins_s, calls: int = 200):
     hp, d = w.heads_per_rank, w.head_dim
     attn_out = [t.reshape(w.tokens, w.cp * hp, d) for t in ins_o]
     attn_lse = [torch.randn(w.tokens, w.cp * hp, device="cuda") for _ in range(w.cp)]
-    lse_ok = hp % 2 == 0
 
     def per_rank():
         for r in range(w.cp):
@@ -143,7 +143,7 @@ def host_timing(w, ws, ins_o, ins_s, calls: int = 200):
         helix_a2a.dcp_a2a_lse_reduce(attn_out, attn_lse, ws)
 
     out = {}
-    for name, fn in (("alltoall_x_cp", per_rank), ("alltoall_loopback", loopback)) + ((("dcp_a2a_lse_reduce", reduce),) if lse_ok else ()):
+    for name, fn in (("alltoall_x_cp", per_rank), ("alltoall_loopback", loopback), ("dcp_a2a_lse_reduce", reduce)):
         for _ in range(20):
             fn()
         torch.cuda.synchronize()
@@ -158,6 +158,117 @@ def host_timing(w, ws, ins_o, ins_s, calls: int = 200):
                      "p95": percentile(samples, 0.95) * 1e6}
     out["note"] = (f"alltoall_x_cp = {w.cp} calls of helix_a2a.alltoall (the reference's signature), one per logical rank; "
                    "each figure is the wall time of the Python call(s) alone, GPU idle before and drained after")
+    return out
+
+
+def _event_us(fn, steps: int, warmup: int) -> float:
+    """HIP-event time of `steps` back-to-back calls of fn on the current stream, per call, in microseconds."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(steps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / steps * 1e3
+
+
+def _graph_of(fn, calls: int):
+    """`calls` invocations of fn captured into one HIP graph (after a few eager ones: lazy set-up stays outside)."""
+    import torch
+
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        keep = [fn() for _ in range(calls)]
+    torch.cuda.synchronize()
+    return graph, keep
+
+
+GRAPH_CALLS = 10  # exchanges per captured graph in the per-rank and decode-size rows: amortises the cost of a graph launch
+
+
+def per_rank_gpu_timing(names=("c2", "c3"), steps: int = 200, spare=None):
+    """GPU time of the reference's signature: cp calls of helix_a2a.alltoall (one per logical rank) per exchange,
+    beside the one fused call of all ranks. HIP events around back-to-back exchanges; `eager` is bounded below
+    by what the Python calls cost the host, `graph` replays a captured graph of GRAPH_CALLS exchanges.
+    `spare` = (workload name, workspace) already allocated by the caller."""
+    import torch
+
+    import helix_a2a
+    from helix_a2a import _ops
+    from helix_workloads import WORKLOADS, make_inputs
+
+    out = {"unit": "us per exchange of all ranks", "graph_calls": GRAPH_CALLS}
+    for name in names:
+        w = WORKLOADS[name]
+        if spare is not None and spare[0] == name:
+            ws = spare[1]
+        else:
+            ws = helix_a2a.allocate_workspace(w.cp, 0)
+            for r in range(w.cp):
+                helix_a2a.init_workspace(ws, r, w.cp)
+        ins_o, ins_s = make_inputs(w, "cuda")
+        plan = _ops.LoopbackPlan(ins_o, ins_s, ws)
+
+        def per_rank():
+            return [helix_a2a.alltoall(ins_o[r], ins_s[r], ws, r, w.cp) for r in range(w.cp)]
+
+        row = {"loopback": {"eager": _event_us(plan.run, steps, 30)}}
+        graph, keep = _graph_of(plan.run, GRAPH_CALLS)
+        row["loopback"]["graph"] = _event_us(graph.replay, max(steps // GRAPH_CALLS, 10), 3) / GRAPH_CALLS
+        del graph, keep
+        for policy, eager_send in (("alltoall_x_cp", False), ("alltoall_x_cp_eager_send", True)):
+            _ops.set_eager_send(eager_send)
+            try:
+                row[policy] = {"eager": _event_us(per_rank, steps, 30)}
+                graph, keep = _graph_of(per_rank, GRAPH_CALLS)
+                row[policy]["graph"] = _event_us(graph.replay, max(steps // GRAPH_CALLS, 10), 3) / GRAPH_CALLS
+                del graph, keep
+            finally:
+                _ops.set_eager_send(False)
+        row["alltoall_x_cp_over_loopback"] = {k: row["alltoall_x_cp"][k] / row["loopback"][k] for k in ("eager", "graph")}
+        out[name] = row
+        torch.cuda.synchronize()
+        del plan, ins_o, ins_s, ws
+    out["note"] = ("alltoall_x_cp: the default, in which the last rank's call issues the exchange of all ranks as one fused "
+                   "launch; alltoall_x_cp_eager_send: HELIX_A2A_EAGER_SEND=1, every rank's send half is a launch of its own "
+                   "at its call (cp send launches + 1 receive launch, one after the other on the stream)")
+    return out
+
+
+def decode_size_timing(names=("c1", "c2", "c5b"), steps: int = 400):
+    """The small workloads, where a Python loop launches slower than the kernels run: the exchange and the
+    exchange fused with the combine replayed from a HIP graph of GRAPH_CALLS calls, per call."""
+    import torch
+
+    import helix_a2a
+    from helix_a2a import _ops
+    from helix_workloads import WORKLOADS, make_inputs
+
+    out = {"unit": "us per call, HIP graph of %d calls replayed back to back" % GRAPH_CALLS}
+    for name in names:
+        w = WORKLOADS[name]
+        ws = helix_a2a.allocate_workspace(w.cp, 0)
+        for r in range(w.cp):
+            helix_a2a.init_workspace(ws, r, w.cp)
+        ins_o, ins_s = make_inputs(w, "cuda")
+        row = {}
+        for kind, plan in (("exchange", _ops.LoopbackPlan(ins_o, ins_s, ws)),
+                           ("exchange_combine", _ops.CombinePlan(ins_o, ins_s, ws, _ops.STATS_MAX_SUM, False, 0))):
+            graph, keep = _graph_of(plan.run, GRAPH_CALLS)
+            row[kind] = _event_us(graph.replay, max(steps // GRAPH_CALLS, 10), 3) / GRAPH_CALLS
+            row[kind + "_eager"] = _event_us(plan.run, steps, 30)
+            del graph, keep
+        out[name] = row
+        torch.cuda.synchronize()
+        del ws
     return out
 
 
@@ -267,7 +378,7 @@ def main() -> int:
 
     import helix_a2a
     from helix_a2a import _ops
-    from helix_a2a.workloads import WORKLOADS, as_head_layout, make_inputs
+    from helix_workloads import WORKLOADS, as_head_layout, make_inputs
     from oracle import helix_oracle as ho
 
     if not torch.cuda.is_available():
@@ -340,6 +451,14 @@ def main() -> int:
     status = _ops.device_status()
     avg_kernel_ms = region_start.elapsed_time(region_end) / args.steps  # launch-to-launch, gaps included
     ms_per_step = wall * 1e3 / args.steps
+    # The roofline legs want a window long enough to average over: a run with fewer than MIN_ROOFLINE_STEPS
+    # timed steps (20 steps of c3 are half a millisecond) times them over a region of their own. `value` and
+    # `ms_per_step` stay on exactly --steps steps.
+    roofline_steps = max(args.steps, MIN_ROOFLINE_STEPS)
+    if graph is not None:
+        roofline_steps = args.steps
+    if roofline_steps != args.steps:
+        avg_kernel_ms = _event_us(plan.run, roofline_steps, 0) * 1e-3
 
     # distribution of single calls (event pair per call), outside the timed region
     n_dist = min(args.steps, 500)
@@ -368,15 +487,15 @@ def main() -> int:
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         cold_start.record()
-        for i in range(args.steps):
+        for i in range(roofline_steps):
             plans[i % n_sets].run()
         cold_end.record()
         torch.cuda.synchronize()
         cold_wall = time.perf_counter() - t0
         status |= _ops.device_status()
-        cold = {"sets": n_sets, "tensor_bytes_in_rotation": n_sets * tensor_bytes,
-                "kernel_us": cold_start.elapsed_time(cold_end) / args.steps * 1e3,
-                "us_per_call": cold_wall * 1e6 / args.steps}
+        cold = {"sets": n_sets, "tensor_bytes_in_rotation": n_sets * tensor_bytes, "steps": roofline_steps,
+                "kernel_us": cold_start.elapsed_time(cold_end) / roofline_steps * 1e3,
+                "us_per_call": cold_wall * 1e6 / roofline_steps}
         del plans
 
     ok = status == 0
@@ -451,6 +570,7 @@ def main() -> int:
         "roofline": {
             "bound": "hbm",
             "kernel": kernel_name,
+            "steps": roofline_steps,  # launches the event-timed region of `achieved` (and of the cold leg) covers
             "achieved": achieved,
             "peak": PEAK_HBM_GBPS,
             "unit": "GB/s",
@@ -468,6 +588,9 @@ def main() -> int:
     if not args.no_host_timing and not args.combine and args.layout == "token" and graph is None:
         result["host_us_per_call"] = host_timing(w, ws, ins_o, ins_s)
         result["memory_probe"] = memory_probe()
+        del plan
+        result["per_rank_gpu_us"] = per_rank_gpu_timing(spare=(w.name, ws))
+        result["decode_sizes_us"] = decode_size_timing()
     if not args.no_cpu_baseline and not args.combine and args.layout == "token":
         result["cpu_baseline"] = cpu_baseline(w, bytes_per_call)
     print(json.dumps(result))

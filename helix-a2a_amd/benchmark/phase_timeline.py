@@ -21,7 +21,7 @@ from pathlib import Path
 
 HERE = Path(__file__).resolve().parent
 PKG = HERE.parent
-for _p in (PKG,):
+for _p in (PKG, PKG.parent):  # the package, and the repository root (helix_workloads.py)
     if str(_p) not in sys.path:
         sys.path.insert(0, str(_p))
 
@@ -51,7 +51,7 @@ def main() -> int:
 
     import helix_a2a
     from helix_a2a import _ops
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     lib = _ops._lib
     lib.helix_a2a_timeline_read.argtypes = [ctypes.c_void_p, ctypes.c_int]

@@ -82,6 +82,7 @@ struct DeviceState {
   uint8_t* scratch = nullptr;  // this device's copy of the built-in workspace (helix_a2a_alltoall_loopback_static)
   std::mutex scratchMutex;
   int scratchCp = 0;           // cp_size the built-in workspace is laid out and initialised for (0 = not yet)
+  bool scratchInGraphs = false;  // a call on the built-in workspace was captured: replays lay it out behind the host's back
 };
 DeviceState g_devices[kMaxDevices];
 
@@ -365,12 +366,16 @@ int launch_rounds(Plan& plan, bool send, bool recv, bool allowRounds, hipStream_
   return HELIX_A2A_OK;
 }
 
-// Wait for `stream`, read the device status word and clear it.
+// Wait for `stream`, read the device status word and clear it. Everything is ordered on `stream` itself (nothing
+// goes through the legacy default stream, which may not be touched while some other stream is being captured).
 int read_status(DeviceState* st, hipStream_t stream, uint32_t* out) {
-  HELIX_HIP_TRY(hipStreamSynchronize(stream));
   uint32_t host = 0;
-  HELIX_HIP_TRY(hipMemcpy(&host, st->status, sizeof(host), hipMemcpyDeviceToHost));
-  if (host != 0) HELIX_HIP_TRY(hipMemset(st->status, 0, sizeof(uint32_t)));
+  HELIX_HIP_TRY(hipMemcpyAsync(&host, st->status, sizeof(host), hipMemcpyDeviceToHost, stream));
+  HELIX_HIP_TRY(hipStreamSynchronize(stream));
+  if (host != 0) {
+    HELIX_HIP_TRY(hipMemsetAsync(st->status, 0, sizeof(uint32_t), stream));
+    HELIX_HIP_TRY(hipStreamSynchronize(stream));
+  }
   *out = host;
   return HELIX_A2A_OK;
 }
@@ -494,8 +499,14 @@ int helix_a2a_alltoall_loopback_static(const helix_a2a_params_t* per_rank, int c
     // The array keeps the last call's contents. Its layout depends on cp_size, so a change of cp_size
     // (or the first call, or a caller's request) lays it out again: FIFO bytes 0xFF, counters 0, by a
     // fill kernel in stream order ahead of the exchange.
+    // A captured call always records the fill kernels: whatever ran on the array between two replays of the
+    // graph, every replay starts from a layout of its own. From then on the host no longer knows what layout
+    // the array holds when an eager call arrives, so eager calls lay it out every time as well.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    const bool capturing = hipStreamIsCapturing(s, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone;
     std::lock_guard<std::mutex> lock(st->scratchMutex);
-    if (reset || st->scratchCp != cp_size) {
+    if (capturing) st->scratchInGraphs = true;
+    if (reset || st->scratchInGraphs || st->scratchCp != cp_size) {
       for (int r = 0; r < cp_size; ++r)
         HELIX_HIP_TRY(launch_init_row(ws.base + static_cast<uint64_t>(r) * ws.rowStrideBytes,
                                       fifo_region_bytes(cp_size, ws.maxChannels),

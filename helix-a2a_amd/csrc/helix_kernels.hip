@@ -183,6 +183,7 @@ __device__ __forceinline__ void report_broken(const KernelArgs& a, int lane) {
 // runs of several passes: the same bytes move in more, shorter wavefronts without one more counter.
 struct TeamLds {
   int64_t step;
+  int bad;  // a wavefront of the team met a corrupt line: the leader leaves the stream's counters where they are
 };
 // A barrier of the workgroup that waits for this wavefront's LDS traffic only (not, as __syncthreads
 // does, for its outstanding loads and stores to memory).
@@ -193,6 +194,11 @@ __device__ __forceinline__ int64_t team_share_step(TeamLds* lds, bool leader, in
   team_barrier();
   return *reinterpret_cast<volatile int64_t*>(&lds->step);
 }
+// A wavefront of a team that met a corrupt line says so before the team's next barrier; the leader looks after it.
+__device__ __forceinline__ void team_report_bad(TeamLds* lds, int lane) {
+  if (lane == 0) *reinterpret_cast<volatile int*>(&lds->bad) = 1;
+}
+__device__ __forceinline__ bool team_is_bad(TeamLds* lds) { return *reinterpret_cast<volatile int*>(&lds->bad) != 0; }
 
 // Every scalar of the argument block a wavefront needs before its first memory access, asked for at once:
 // the compiler then fetches the block in a few wide scalar loads and one wait at the top of the kernel,
@@ -442,7 +448,9 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
     step = *mine;
     head = ld_counter(token);
     broken = broken_at_launch(a) != 0;
+    if (kTeam && lane == 0) *reinterpret_cast<volatile int*>(&lds->bad) = 0;  // ahead of the team's first barrier
   }
+  bool corrupt = false;  // this wavefront met a line whose flag disagrees with the token: it stores nothing from then on
 
   for (int firstMsg = 0; firstMsg < st.msgs; firstMsg += st.msgsPerEntry) {
     const int runMsgs = min(st.msgsPerEntry, st.msgs - firstMsg);
@@ -482,7 +490,7 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
     } else {
       if (firstMsg > 0) team_barrier();  // every wavefront of the team has its lines of the previous entry in registers
       bool ok = true;
-      if (leader) ok = leader_acquires();
+      if (leader) ok = !team_is_bad(lds) && leader_acquires();  // after a corrupt line the team leaves, counters untouched
       step = team_share_step(lds, leader, lane, ok ? step : -1);
       if (step < 0) return;
     }
@@ -508,14 +516,18 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
       }
       if (__ballot(!flagsAgree) != 0ull) {
         raise_status(a, kStatusInternal, lane);
-        if (!kTeam) return;  // a wavefront of a team stays with its team to the last barrier; the workspace is marked broken
+        if (!kTeam) return;
+        // a wavefront of a team stays with its team to the next barrier, where the leader learns of it; it
+        // stores nothing any more, and the workspace is marked broken
+        if (!corrupt) team_report_bad(lds, lane);
+        corrupt = true;
       }
       if (U0 == slice.begin && firstMsg == 0) HELIX_MARK(wave, 1, false);
 #pragma unroll
       for (int i = 0; i < kUnitsInFlight; ++i) {
         uint32_t U = U0 + i * kWaveLanes + lane;
         RunUnit d;
-        UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < passEnd, &d);
+        UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < passEnd && !(kTeam && corrupt), &d);
         u32x2 wa = {v[i].x, v[i].y};
         u32x2 wb = {v[i].z, v[i].w};
         if (kAlignedStores) {
@@ -576,6 +588,7 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
   }
   HELIX_MARK(wave, 2, false);
   if (kTeam) team_barrier();  // every wavefront of the team has the lines of the last entry in registers
+  if (kTeam && leader && team_is_bad(lds)) return;
   if (leader && lane == 0) {  // close the last entry (csrc/helix_alltoall.cu:468-472)
     st_counter(mine, step + 1);
     if (counterPart == 0) st_counter(&senderInfo[1], step + 1);

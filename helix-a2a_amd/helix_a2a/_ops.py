@@ -15,7 +15,6 @@ import ctypes
 import os
 import threading
 import time
-import weakref
 from pathlib import Path
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -131,7 +130,8 @@ def _require(cond: bool, msg: str) -> None:
 
 
 def _stream_handle() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """The current stream of the current device as a raw hipStream_t (no Python stream object is built)."""
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
 
 
 # --------------------------------------------------------------------------
@@ -172,7 +172,7 @@ class _on_device:
 
     def __init__(self, device: torch.device) -> None:
         index = device.index
-        self.ctx = None if index is None or index == torch.cuda.current_device() else torch.cuda.device(device)
+        self.ctx = None if index is None or index == torch._C._cuda_getDevice() else torch.cuda.device(device)
 
     def __enter__(self):
         if self.ctx is not None:
@@ -202,8 +202,9 @@ def initialize_workspace(workspace: torch.Tensor, cp_rank: int, cp_size: int) ->
     row_ptr = workspace.data_ptr() + cp_rank * workspace.stride(0) * 8
     # a reset starts a new epoch: half-finished exchanges of logical ranks on this workspace are void
     with _call_lock:
-        _groups.pop((workspace.device.index or 0, workspace.data_ptr(), cp_size), None)
-    _reduce_descriptors.clear()
+        _groups.pop((workspace.data_ptr(), cp_size), None)
+    with _reduce_lock:
+        _reduce_descriptors.clear()
     with torch.cuda.device(workspace.device):
         _check(_lib.helix_a2a_init_workspace(row_ptr, cp_size, 0, _stream_handle()), "init_workspace")
 
@@ -330,7 +331,7 @@ class _ExchangeShape:
 
 
 _shapes: Dict[tuple, _ExchangeShape] = {}
-_call_lock = threading.RLock()  # the cached descriptor arrays are rewritten by every call
+_call_lock = threading.Lock()  # the cached descriptor arrays are rewritten by every call
 
 
 def _exchange_shape(partial_o: torch.Tensor, softmax_stats: torch.Tensor, cp_size: int) -> _ExchangeShape:
@@ -373,103 +374,146 @@ def set_pending_expiry(seconds: float) -> None:
     _PENDING_EXPIRY_S = float(seconds)
 
 
+def _env_flag(name: str) -> bool:
+    return os.environ.get(name, "") not in ("", "0")
+
+
+_eager_send = _env_flag("HELIX_A2A_EAGER_SEND")
+
+
+def set_eager_send(enabled: bool) -> None:
+    """When a logical rank's send half is enqueued by :func:`alltoall_native` (process-wide; takes effect with
+    the next exchange that starts).
+
+    ``False`` (default): with the last rank's call, as one fused launch of all ranks -- the exchange then costs
+    what ``alltoall_loopback`` costs. A rank's inputs belong to the exchange until every rank has called, as
+    its outputs do.
+    ``True``: at once, on the caller's stream, one launch per rank (the receive halves still follow the last
+    rank's call). The caller may overwrite a rank's inputs in stream order right after that rank's call, as
+    with the reference; the ``cp_size`` send launches run one after the other. ``HELIX_A2A_EAGER_SEND=1``
+    switches it on from the start.
+    """
+    global _eager_send
+    _eager_send = bool(enabled)
+
+
 class _LogicalRankGroup:
     """The ranks of one workspace that share this device.
 
-    A rank's call enqueues its send half at once. Its receive half depends on
-    every peer's send half, so it is enqueued when the last rank of the group
-    has called: from then on stream order guarantees the lines are in the FIFOs.
-    The tensors are kept alive here until that launch.
+    A rank's receive half depends on every peer's send half, so nothing can complete before the last rank of
+    the group has called. By default the whole exchange is therefore issued by that call, as one fused launch
+    of all ranks on the last caller's stream; until then the group keeps the ranks' tensors (and the
+    workspace) alive, and a rank must leave its inputs alone. With ``set_eager_send(True)`` a rank's call
+    enqueues its send half at once and only the receive halves wait for the last rank -- unless the exchange
+    is too large for the four FIFO entries of a stream (a send launch cannot be back-pressured by a receive
+    launch queued behind it), which falls back to the fused launch and its stream-ordered rounds.
 
-    An exchange too large for the four FIFO entries of a stream cannot send
-    ahead of its receivers; its send halves are held back as well and the last
-    rank's call issues everything as one loopback exchange, which splits into
-    stream-ordered rounds (then a rank must leave its inputs alone until every
-    rank has called).
+    The outputs of all ranks are two allocations made by the first rank's call; every rank is handed its slice.
 
-    The channel count of an exchange (HELIX_A2A_CHANNEL_COUNT or automatic) is
-    settled by its first rank's call and used for every launch of it, whatever
-    the environment says later.
+    The channel count of an exchange (HELIX_A2A_CHANNEL_COUNT or automatic) is settled by its first rank's
+    call and used for every launch of it, whatever the environment says later.
     """
+
+    __slots__ = ("cp_size", "pending", "streams", "shape", "arr", "eager", "started", "workspace", "outs_o", "outs_s")
 
     def __init__(self, cp_size: int) -> None:
         self.cp_size = cp_size
-        self.pending: Dict[int, Tuple[tuple, torch.cuda.Stream]] = {}
-        self.shape: Optional[_ExchangeShape] = None
-        self.arr: Optional[ctypes.Array] = None
-        self.deferred = False
-        self.started = 0.0
+        self.pending: Dict[int, tuple] = {}   # rank -> the tensors of its call
+        self.streams: Dict[int, int] = {}     # rank -> raw stream handle it called on
+        self._forget()
 
     def _forget(self) -> None:
         self.pending.clear()
-        self.shape = None
-        self.arr = None
-        self.deferred = False
+        self.streams.clear()
+        self.shape: Optional[_ExchangeShape] = None
+        self.arr: Optional[ctypes.Array] = None
+        self.eager = False
+        self.started = 0.0
+        self.workspace: Optional[torch.Tensor] = None
+        self.outs_o = self.outs_s = None
+
+    def _begin(self, shape: _ExchangeShape, workspace: torch.Tensor) -> None:
+        channels = _env_channel_count()
+        max_ch = _device_max_channels(self.cp_size)
+        _require(channels <= max_ch, f"alltoall: channel_count {channels} exceeds max_channel_count {max_ch}")
+        self.shape = shape
+        self.arr = shape.array(workspace, channels)
+        self.eager = _eager_send
+        self.started = time.monotonic()
+        self.workspace = workspace  # kept while ranks are pending: the caller may have passed a temporary view
+        device = workspace.device
+        self.outs_o = torch.empty((self.cp_size,) + tuple(shape.shape_o), dtype=shape.dtype, device=device).unbind(0)
+        self.outs_s = torch.empty((self.cp_size,) + tuple(shape.shape_s), dtype=torch.float32, device=device).unbind(0)
 
     def submit(self, rank: int, shape: _ExchangeShape, workspace: torch.Tensor, partial_o: torch.Tensor,
-               softmax_stats: torch.Tensor, out_o: torch.Tensor, out_s: torch.Tensor) -> None:
-        if self.pending and time.monotonic() - self.started > _PENDING_EXPIRY_S:
-            waited = sorted(self.pending)
-            self._forget()
-            raise RuntimeError(f"logical ranks {waited} waited more than {_PENDING_EXPIRY_S:.0f} s for the other ranks of "
-                               "their exchange; it is given up: re-initialise the workspace before the next exchange")
-        if rank in self.pending:
-            raise RuntimeError(f"logical rank {rank} called alltoall again before all {self.cp_size} ranks of the group had called")
-        if self.pending:
+               softmax_stats: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        pending = self.pending
+        if pending:
+            if time.monotonic() - self.started > _PENDING_EXPIRY_S:
+                waited = sorted(pending)
+                self._forget()
+                raise RuntimeError(f"logical ranks {waited} waited more than {_PENDING_EXPIRY_S:.0f} s for the other ranks of "
+                                   "their exchange; it is given up: re-initialise the workspace before the next exchange")
+            if rank in pending:
+                raise RuntimeError(f"logical rank {rank} called alltoall again before all {self.cp_size} ranks of the group had called")
             _require(shape is self.shape, "logical ranks of one group must exchange tensors of one shape and dtype")
         else:
-            self.shape = shape
-            self.arr = shape.array(workspace, _env_channel_count())
-            self.deferred = False
-            self.started = time.monotonic()
+            self._begin(shape, workspace)
+        out_o, out_s = self.outs_o[rank], self.outs_s[rank]
         p = self.arr[rank]
         p.send_fields[0].data = partial_o.data_ptr()
         p.send_fields[1].data = softmax_stats.data_ptr()
         p.recv_fields[0].data = out_o.data_ptr()
         p.recv_fields[1].data = out_s.data_ptr()
-        stream = torch.cuda.current_stream()
-        if not self.deferred:
-            rc = _lib.helix_a2a_alltoall_send(ctypes.byref(p), 1, stream.cuda_stream)
-            if rc == 3 and not self.pending:  # HELIX_A2A_ERR_CAPACITY on the first rank: hold everything back
-                self.deferred = True
+        stream = _stream_handle()
+        if self.eager:
+            rc = _lib.helix_a2a_alltoall_send(ctypes.byref(p), 1, stream)
+            if rc == 3 and not pending:  # HELIX_A2A_ERR_CAPACITY on the first rank: the fused launch and its rounds instead
+                self.eager = False
             elif rc != 0:
-                if not self.pending:
+                if not pending:
                     self._forget()
                 _raise_last("alltoall (send half)")
-        self.pending[rank] = ((partial_o, softmax_stats, out_o, out_s), stream)
-        if len(self.pending) == self.cp_size:
+        pending[rank] = (partial_o, softmax_stats)
+        self.streams[rank] = stream
+        if len(pending) == self.cp_size:
             self._flush(stream)
+        return out_o, out_s
 
-    def _flush(self, stream: torch.cuda.Stream) -> None:
+    def _flush(self, stream: int) -> None:
         """Enqueue what is left of the exchange on the last caller's stream.
 
-        That stream first waits for the work of every other stream a rank called
-        on (its send half, or the producer of its inputs); afterwards those
-        streams wait for this launch, so each rank's outputs are valid once the
-        stream *it* called on has drained.
+        That stream first waits for the work of every other stream a rank called on (its send half, or the
+        producer of its inputs); afterwards those streams wait for this launch, so each rank's outputs are
+        valid once the stream *it* called on has drained.
         """
-        others = {s.cuda_stream: s for _k, s in self.pending.values() if s.cuda_stream != stream.cuda_stream}
         try:
-            for other in others.values():
-                ev = torch.cuda.Event()
-                ev.record(other)
-                stream.wait_event(ev)
-            if self.deferred:
-                rc = _lib.helix_a2a_alltoall_loopback(self.arr, self.cp_size, stream.cuda_stream)
+            others = set(self.streams.values())
+            others.discard(stream)
+            mine = None
+            if others:
+                mine = torch.cuda.ExternalStream(stream)
+                others = [torch.cuda.ExternalStream(h) for h in others]
+                for other in others:
+                    ev = torch.cuda.Event()
+                    ev.record(other)
+                    mine.wait_event(ev)
+            if self.eager:
+                rc = _lib.helix_a2a_alltoall_recv(self.arr, self.cp_size, stream)
             else:
-                rc = _lib.helix_a2a_alltoall_recv(self.arr, self.cp_size, stream.cuda_stream)
+                rc = _lib.helix_a2a_alltoall_loopback(self.arr, self.cp_size, stream)
             if rc != 0:
-                _raise_last("alltoall (receive half)")
+                _raise_last("alltoall (receive half)" if self.eager else "alltoall")
             if others:
                 done = torch.cuda.Event()
-                done.record(stream)
-                for other in others.values():
+                done.record(mine)
+                for other in others:
                     other.wait_event(done)
         finally:
             self._forget()
 
 
-_groups: Dict[Tuple[int, int, int], _LogicalRankGroup] = {}
+_groups: Dict[Tuple[int, int], _LogicalRankGroup] = {}  # (workspace address, cp_size) -> its logical ranks
 
 
 def reset_logical_ranks() -> None:
@@ -478,9 +522,15 @@ def reset_logical_ranks() -> None:
         _groups.clear()
 
 
-def _drop_group(key: Tuple[int, int, int]) -> None:
-    with _call_lock:
-        _groups.pop(key, None)
+def _group_of(workspace: torch.Tensor, cp_size: int) -> _LogicalRankGroup:
+    key = (workspace.data_ptr(), cp_size)
+    group = _groups.get(key)
+    if group is None:
+        if len(_groups) >= 64:  # groups between exchanges hold nothing worth keeping
+            for k in [k for k, g in _groups.items() if not g.pending]:
+                del _groups[k]
+        group = _groups[key] = _LogicalRankGroup(cp_size)
+    return group
 
 
 def alltoall_native(partial_o: torch.Tensor, softmax_stats: torch.Tensor, workspace: torch.Tensor,
@@ -488,20 +538,14 @@ def alltoall_native(partial_o: torch.Tensor, softmax_stats: torch.Tensor, worksp
     """One logical rank's exchange; see :func:`helix_a2a.alltoall`."""
     _require(1 <= cp_size <= MAX_CP_SIZE, f"cp_size must be in [1, {MAX_CP_SIZE}]")
     shape = _exchange_shape(partial_o, softmax_stats, cp_size)
-    _check_workspace(workspace, cp_size)
+    if not (isinstance(workspace, torch.Tensor) and workspace.dtype is torch.int64 and workspace.dim() == 2
+            and workspace.size(0) == cp_size and workspace.stride(1) == 1 and workspace.is_cuda):
+        _check_workspace(workspace, cp_size)  # says which of them it was
     _require(0 <= cp_rank < cp_size, "cp_rank must be in [0, cp_size)")
-    _require(workspace.device == partial_o.device == softmax_stats.device, "all tensors must live on one device")
-    out_o = torch.empty_like(partial_o)
-    out_s = torch.empty_like(softmax_stats)
-    with _call_lock, _on_device(partial_o.device):
-        key = (workspace.device.index or 0, workspace.data_ptr(), cp_size)
-        group = _groups.get(key)
-        if group is None:
-            group = _groups[key] = _LogicalRankGroup(cp_size)
-            # nothing is left waiting on a workspace that no longer exists
-            weakref.finalize(workspace, _drop_group, key)
-        group.submit(cp_rank, shape, workspace, partial_o, softmax_stats, out_o, out_s)
-    return out_o, out_s
+    device = workspace.device
+    _require(device == partial_o.device and device == softmax_stats.device, "all tensors must live on one device")
+    with _call_lock, _on_device(device):
+        return _group_of(workspace, cp_size).submit(cp_rank, shape, workspace, partial_o, softmax_stats)
 
 
 def alltoall_loopback(partial_o: Sequence[torch.Tensor], softmax_stats: Sequence[torch.Tensor],
@@ -731,44 +775,40 @@ def dcp_reduce(cp_attn_out: Sequence[torch.Tensor], cp_attn_lse: Sequence[torch.
     _check_workspace(workspace, n)
     _require(workspace.device == device, "all tensors must live on one device")
     key = (n, b, h, d, dtype, workspace.data_ptr(), workspace.stride(0), int(channel_count), device.index)
-    with _reduce_lock:
+    # one allocation per kind of output; rank r's result is slice r of it
+    combined = torch.empty((n, b, hp, d), dtype=dtype, device=device).unbind(0)
+    lses = torch.empty((n, b, hp), dtype=torch.float32, device=device).unbind(0) if return_lse else None
+    keep = []
+    with _reduce_lock, _on_device(device):
         desc = _reduce_descriptors.get(key)
         if desc is None:
             if len(_reduce_descriptors) >= 64:
                 _reduce_descriptors.clear()
             desc = _reduce_descriptors[key] = _ReduceDescriptors(n, b, h, d, dtype, workspace, channel_count)
-    combined: List[torch.Tensor] = []
-    lses: Optional[List[torch.Tensor]] = [] if return_lse else None
-    keep = []
-    with _reduce_lock, _on_device(device):
+        arr, out = desc.arr, desc.out
         for r in range(n):
             o, lse = cp_attn_out[r], cp_attn_lse[r]
-            _require(o.shape == shape and o.dtype == dtype and o.device == device,
-                     "all ranks must pass cp_attn_out of one shape, dtype and device")
-            _require(lse.shape == lse_shape and lse.dtype == torch.float32 and lse.device == device,
-                     "cp_attn_lse must be float32 [B, H] on the same device")
+            if not (o.shape == shape and o.dtype == dtype and o.device == device):
+                raise RuntimeError("all ranks must pass cp_attn_out of one shape, dtype and device")
+            if not (lse.shape == lse_shape and lse.dtype == torch.float32 and lse.device == device):
+                raise RuntimeError("cp_attn_lse must be float32 [B, H] on the same device")
             if not o.is_contiguous():
                 o = o.contiguous()
+                keep.append(o)
             if not lse.is_contiguous():
                 lse = lse.contiguous()
-            keep.append((o, lse))
-            c = torch.empty((b, hp, d), dtype=dtype, device=device)
-            combined.append(c)
-            p = desc.arr[r]
-            p.send_fields[0].data = o.data_ptr()
-            p.send_fields[1].data = lse.data_ptr()
-            desc.out[r].combined = c.data_ptr()
-            if return_lse:
-                lo = torch.empty((b, hp), dtype=torch.float32, device=device)
-                lses.append(lo)
-                desc.out[r].lse_out = lo.data_ptr()
-            else:
-                desc.out[r].lse_out = None
+                keep.append(lse)
+            fields = arr[r].send_fields
+            fields[0].data = o.data_ptr()
+            fields[1].data = lse.data_ptr()
+            out[r].combined = combined[r].data_ptr()
+            out[r].lse_out = lses[r].data_ptr() if return_lse else None
         mode = STATS_LSE_PACKED | (STATS_BASE2 if lse_base2 else 0)
-        rc = _lib.helix_a2a_alltoall_combine_loopback(desc.arr, desc.out, n, mode, desc.dtype_code, _stream_handle())
+        rc = _lib.helix_a2a_alltoall_combine_loopback(arr, out, n, mode, desc.dtype_code, _stream_handle())
     if rc != 0:
         _raise_last("dcp_a2a_lse_reduce")
-    return (combined, lses) if return_lse else combined
+    combined = list(combined)
+    return (combined, list(lses)) if return_lse else combined
 
 
 def device_status() -> int:

@@ -4,7 +4,8 @@ Each workload describes one decode step of ``cp`` context-parallel ranks:
 every rank holds ``partial_o [T, cp, H/cp, D]`` (bf16) and
 ``softmax_stats [T, cp, H/cp, 2]`` (fp32 pairs of running max and running
 sum). Through the 3-D API they are passed as ``[T, cp, (H/cp)*D]`` and
-``[T, cp, 2*H/cp]``. The same shapes drive the tests and the benchmark.
+``[T, cp, 2*H/cp]``. The same shapes drive the tests and the benchmark; the
+module is test and benchmark equipment, not part of the ``helix_a2a`` package.
 """
 from __future__ import annotations
 

@@ -170,6 +170,13 @@ int helix_a2a_alltoall(const helix_a2a_params_t* params, void* stream);
  * back-pressured by a receive launch queued behind it.
  * Same reference counterpart as helix_a2a_alltoall (the sender branch,
  * csrc/helix_alltoall.cu:360-412, and the receiver branch, :413-473).
+ * Order: the send launch of an exchange must have completed, or be ordered
+ * ahead of its receive launch on one stream or by events, and the receive
+ * launch of one exchange ahead of the send launch of the next on the same
+ * workspace. When a stream's runs are shared by several wavefronts (see
+ * helix_a2a_set_units_per_wavefront) only the first of them keeps the counter
+ * that senders wait on for FIFO room, so halves that run unordered beside each
+ * other could overwrite an entry that is still being read.
  */
 int helix_a2a_alltoall_send(const helix_a2a_params_t* per_rank, int rank_count, void* stream);
 int helix_a2a_alltoall_recv(const helix_a2a_params_t* per_rank, int rank_count, void* stream);
@@ -205,6 +212,12 @@ int helix_a2a_alltoall_loopback(const helix_a2a_params_t* per_rank, int cp_size,
  *   races   all calls on one GPU share that GPU's array: they must be ordered
  *           with respect to each other (one stream, or events). Calls that
  *           overlap on one GPU race.
+ *   capture a call recorded into a graph always records the fill kernels too,
+ *           so that every replay lays the array out for itself whatever ran on it
+ *           in between; after the first such capture on a device, eager calls on
+ *           that device lay the array out on every call as well (the host cannot
+ *           know what a replay left behind). Checked mode does nothing on a
+ *           capturing stream.
  * The very first library call on a device performs the one-time set-up
  * (device query, symbol addresses); make any library call before starting a
  * graph capture.
@@ -239,7 +252,10 @@ int helix_a2a_device_status(uint32_t* status, void* stream);
  * -- the rest of the launch and every launch queued behind it -- writes nothing
  * and raises HELIX_A2A_STATUS_BROKEN_WORKSPACE, so the output tensors of
  * such an exchange keep whatever they held before; the FIFO counters are no
- * longer consistent. helix_a2a_init_workspace on row 0 (with the other rows)
+ * longer consistent. (Where the wavefronts of a workgroup walk a run as a team,
+ * the one that met the corrupt line stores nothing from that pass on, its
+ * team-mates finish the pass they are in, and the stream's counters stay where
+ * they were.) helix_a2a_init_workspace on row 0 (with the other rows)
  * makes the workspace usable again. The calls themselves return at launch, so
  * a caller learns of a failure from helix_a2a_device_status, or at once in
  * checked mode:
@@ -250,6 +266,11 @@ int helix_a2a_device_status(uint32_t* status, void* stream);
  * calls synchronous. A call on a stream that is being captured into a graph
  * cannot wait and skips the check. Default 0. The environment variable
  * HELIX_A2A_CHECKED=1 switches it on from the start.
+ * The status word is one per device, and reading it clears it: with exchanges
+ * in flight from several host threads (or on several workspaces) a reader may
+ * take the bits another exchange raised. Checked mode and
+ * helix_a2a_device_status are meant for one thread of control per device; the
+ * broken word, which stops the exchanges behind a failure, is per workspace.
  */
 void helix_a2a_set_checked_mode(int enabled);
 

@@ -73,7 +73,7 @@ def check(combined, lse, want, dtype):
 
 @pytest.mark.parametrize("name", ["c1", "c2", "c5b", "c3", "c4", "c5a"])
 def test_combine_workloads(hx, ops, name):
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS[name]
     ws = workspace(hx, w.cp)
@@ -140,7 +140,7 @@ def test_combine_closed_forms(hx, ops):
 
 
 def test_combine_4d_inputs_and_plan_replay(hx, ops):
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS["c2"]
     ws = workspace(hx, w.cp)
@@ -258,7 +258,7 @@ def test_combine_thirty_two_ranks(hx, ops):
 
 def test_combine_while_senders_are_still_writing(hx, ops):
     # few channels: all wavefronts resident at once, the combine half has to wait for its senders
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS["c3"]
     ws = workspace(hx, w.cp)

@@ -43,6 +43,15 @@ def unchecked(ops):
     ops.set_checked_mode(os.environ.get("HELIX_A2A_CHECKED", "") not in ("", "0"))
 
 
+@pytest.fixture(params=[False, True], ids=["fused-at-last-rank", "eager-send"])
+def send_policy(request, ops):
+    """Both ways a per-rank exchange can be issued: all of it with the last rank's call (default), or every
+    rank's send half at its own call."""
+    ops.set_eager_send(request.param)
+    yield request.param
+    ops.set_eager_send(False)
+
+
 def get_workspace(hx, cp, fresh=False):
     """One workspace per cp for the whole module (4.3 GB at cp = 8), initialised on first use."""
     ws = _WORKSPACES.get(cp)
@@ -156,7 +165,7 @@ def test_input_validation(hx):
 
 @pytest.mark.parametrize("name", ["c1", "c2", "c5b", "c3", "c4", "c5a"])
 def test_loopback_workloads(hx, ops, name):
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS[name]
     ws = get_workspace(hx, w.cp)
@@ -171,7 +180,7 @@ def test_loopback_workloads(hx, ops, name):
 def test_exchange_twice_is_the_identity(hx, ops, name):
     # out[r][e, s] = in[s][e, r], so exchanging the result again returns every rank its own input; and the
     # exchange only moves bytes: sums of the 64-bit words (plain and shifted) over all ranks do not change
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS[name]
     ws = get_workspace(hx, w.cp)
@@ -193,7 +202,7 @@ def test_exchange_twice_is_the_identity(hx, ops, name):
 @pytest.mark.parametrize("name", ["c1", "c5b", "c2"])
 def test_loopback_against_reference_model(hx, ops, ref_model, name):
     # the C restatement of the reference kernel, run on the same bits
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS[name]
     ws = get_workspace(hx, w.cp)
@@ -214,7 +223,7 @@ def test_loopback_against_reference_model(hx, ops, ref_model, name):
 @pytest.mark.parametrize("name", ["c2", "c5b", "c3"])
 def test_per_head_layout(hx, ops, name):
     # the layout the serving integration passes: one entry per (token, head), stats are one float2
-    from helix_a2a.workloads import WORKLOADS, as_head_layout, make_inputs
+    from helix_workloads import WORKLOADS, as_head_layout, make_inputs
 
     w = WORKLOADS[name]
     ws = get_workspace(hx, w.cp)
@@ -230,7 +239,7 @@ def test_per_head_layout(hx, ops, name):
 
 @pytest.mark.parametrize("channels", [1, 2, 3, 4, 8, 16, 32, 64, 128, 0])
 def test_channel_sweep(hx, ops, channels):
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS["c3"]
     ws = get_workspace(hx, w.cp)
@@ -242,7 +251,7 @@ def test_channel_sweep(hx, ops, channels):
 
 
 def test_channel_count_limits(hx, ops):
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS["c1"]
     ws = get_workspace(hx, w.cp)
@@ -383,7 +392,7 @@ def test_special_values_survive(hx, ops):
 # ---------------------------------------------------------------------------
 
 def test_repeated_calls_wrap_the_fifo(hx, ops):
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS["c2"]
     ws = get_workspace(hx, w.cp, fresh=True)
@@ -398,7 +407,7 @@ def test_repeated_calls_wrap_the_fifo(hx, ops):
 
 def test_reinit_between_calls(hx, ops):
     # tests/test_mnnvl.py:100-161 re-initialises the workspace before every call
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS["c1"]
     ws = get_workspace(hx, w.cp)
@@ -413,7 +422,7 @@ def test_reinit_between_calls(hx, ops):
 
 def test_many_calls_back_to_back_without_sync(hx, ops):
     # a torn or stale line would show up as a mismatch in one of many asynchronous iterations
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS["c3"]
     ws = get_workspace(hx, w.cp)
@@ -436,7 +445,7 @@ def test_exchange_beside_a_competing_kernel(hx, ops):
     # senders running. Here the device is shared with long unrelated kernels on a second stream of the same
     # (default) priority, which take wavefront slots away from the exchange at arbitrary moments: the
     # exchanges must still complete, bit for bit, with no wait running into its limit.
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS["c3"]
     ws = get_workspace(hx, w.cp)
@@ -471,7 +480,7 @@ def test_exchange_beside_a_competing_kernel(hx, ops):
 # ---------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_per_rank_calls_seeded_full_tensor(hx, ops, dtype):
+def test_per_rank_calls_seeded_full_tensor(hx, ops, dtype, send_policy):
     # tests/test_alltoall.py:303-360 on logical ranks: rank r sends full[:, :, r, :] and receives full[:, r, :, :]
     cp, b, d, s = 4, 4, 128, 2
     ws = get_workspace(hx, cp)
@@ -490,7 +499,7 @@ def test_per_rank_calls_seeded_full_tensor(hx, ops, dtype):
         assert bits_equal(recv_s, full_s[:, rank, :, :])
 
 
-def test_per_rank_calls_fill_vectors(hx, ops):
+def test_per_rank_calls_fill_vectors(hx, ops, send_policy):
     # tests/test_mnnvl.py:164-219: rank r sends the constant r+1; slot j of every result holds j+1
     cp, n, d = 4, 4, 64
     ws = get_workspace(hx, cp)
@@ -509,7 +518,7 @@ def test_per_rank_calls_fill_vectors(hx, ops):
 
 
 def test_per_rank_calls_4d_and_leading_dims(hx, ops):
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS["c2"]
     ws = get_workspace(hx, w.cp)
@@ -527,6 +536,49 @@ def test_per_rank_calls_4d_and_leading_dims(hx, ops):
     torch.cuda.synchronize()
     assert_clean(ops)
     check_against_oracle(ins_o, ins_s, [o[0] for o in outs], [o[1] for o in outs], with_numpy=False)
+
+
+def test_per_rank_calls_with_temporary_workspace_views(hx, ops, send_policy):
+    # every rank hands over a fresh view of the workspace that dies with its call: the exchange must not
+    # be forgotten (nor its workspace freed) between the first rank's call and the last one's
+    cp, entries = 4, 24
+    ws = get_workspace(hx, cp)
+    g = torch.Generator().manual_seed(77)
+    for rep in range(3):
+        ins_o = [torch.randn(entries, cp, 256, generator=g).to(torch.bfloat16).cuda() for _ in range(cp)]
+        ins_s = [torch.randn(entries, cp, 4, generator=g).cuda() for _ in range(cp)]
+        outs = [hx.alltoall(ins_o[r], ins_s[r], ws.view(cp, -1) if r % 2 else ws[:], cp_rank=r, cp_size=cp)
+                for r in range(cp)]
+        torch.cuda.synchronize()
+        assert_clean(ops)
+        check_against_oracle(ins_o, ins_s, [a for a, _ in outs], [b for _, b in outs], with_numpy=False)
+    assert not any(g_.pending for g_ in ops._groups.values())
+
+
+def test_eager_send_lets_a_rank_reuse_its_input_buffer(hx, ops):
+    # with eager sends a rank's inputs are read in stream order at its call, as with the reference: one
+    # buffer refilled for every rank works. (The default issues everything with the last rank's call and
+    # asks the ranks to leave their inputs alone until then.)
+    cp, entries = 4, 32
+    ws = get_workspace(hx, cp)
+    g = torch.Generator().manual_seed(78)
+    ins_o = [torch.randn(entries, cp, 128, generator=g).to(torch.bfloat16).cuda() for _ in range(cp)]
+    ins_s = [torch.randn(entries, cp, 2, generator=g).cuda() for _ in range(cp)]
+    buf_o, buf_s = torch.empty_like(ins_o[0]), torch.empty_like(ins_s[0])
+    ops.set_eager_send(True)
+    try:
+        outs = []
+        for r in range(cp):
+            buf_o.copy_(ins_o[r])
+            buf_s.copy_(ins_s[r])
+            outs.append(hx.alltoall(buf_o, buf_s, ws, cp_rank=r, cp_size=cp))
+        buf_o.zero_()
+        buf_s.zero_()
+    finally:
+        ops.set_eager_send(False)
+    torch.cuda.synchronize()
+    assert_clean(ops)
+    check_against_oracle(ins_o, ins_s, [a for a, _ in outs], [b for _, b in outs], with_numpy=False)
 
 
 def test_per_rank_call_twice_is_an_error(hx, ops):
@@ -684,6 +736,15 @@ def test_corrupt_line_is_reported(hx, ops, teams, unchecked):
         torch.cuda.synchronize()
         status = ops.device_status()
         assert status & ops.STATUS_INTERNAL, status
+        if teams:
+            # 3 messages of 513 pieces on one channel: a run of 103 lines walked by 7 wavefronts, 16 lines each.
+            # The wavefront that owns lines 32..47 (run pieces 480..719: the end of message 0 and pieces 0..206
+            # of message 1) stores nothing; its team-mates store their slices; the stream's counters stay put
+            assert bool((out_o[1][1, 0, :800].view(torch.int16) == 0).all())
+            assert bits_equal(out_o[1][2, 0], o[0][2, 1])
+            max_ch = _max_channels(cp)
+            receiver_info = (512 * 1024 * cp * max_ch + 256 * cp * max_ch) // 8
+            assert int(ws[1, receiver_info + 1]) == 0, "the receiver's counter of the corrupt stream was released"
         hx.alltoall_loopback(o, s, ws, channel_count=channels)
         torch.cuda.synchronize()
         assert ops.device_status() & ops.STATUS_BROKEN_WORKSPACE
@@ -793,7 +854,7 @@ def test_send_capacity_is_checked_for_split_phases(hx, ops):
     assert_clean(ops)
 
 
-def test_per_rank_calls_beyond_fifo_capacity(hx, ops):
+def test_per_rank_calls_beyond_fifo_capacity(hx, ops, send_policy):
     # the reference accepts any entry count (its senders wait for their receivers); per-rank calls of logical
     # ranks hold such an exchange back until the last rank has called and issue it in stream-ordered rounds
     cp, entries = 3, 7300  # one channel: 3612 messages per round
@@ -820,7 +881,7 @@ def test_per_rank_calls_beyond_fifo_capacity(hx, ops):
     check_against_oracle(small_o, small_s, [x[0] for x in results], [x[1] for x in results], with_numpy=False)
 
 
-def test_channel_count_of_an_exchange_is_settled_by_its_first_rank(hx, ops):
+def test_channel_count_of_an_exchange_is_settled_by_its_first_rank(hx, ops, send_policy):
     # the send halves and the receive half of one per-rank exchange are separate launches; the environment
     # may change between them without the halves disagreeing
     cp, entries = 4, 40
@@ -842,7 +903,7 @@ def test_channel_count_of_an_exchange_is_settled_by_its_first_rank(hx, ops):
     check_against_oracle(ins_o, ins_s, [x[0] for x in results], [x[1] for x in results], with_numpy=False)
 
 
-def test_abandoned_per_rank_exchange_expires(hx, ops):
+def test_abandoned_per_rank_exchange_expires(hx, ops, send_policy):
     # a group whose last ranks never call does not pin its tensors for ever: the next call after the expiry
     # time gives the exchange up and says what to do
     cp = 2
@@ -858,20 +919,23 @@ def test_abandoned_per_rank_exchange_expires(hx, ops):
         ops.set_pending_expiry(120.0)
     assert not any(g.pending for g in ops._groups.values())
     torch.cuda.synchronize()
-    for r in range(cp):   # rank 0's lines sit in the FIFOs unreceived
+    for r in range(cp):   # with eager sends rank 0's lines sit in the FIFOs unreceived
         hx.init_workspace(ws, r, cp)
-    # a workspace that goes away takes its group along
+    # a group is found by its workspace's address and rank count
     ws2 = hx.allocate_workspace(cp, 0)
     for r in range(cp):
         hx.init_workspace(ws2, r, cp)
     hx.alltoall(o, s, ws2, 0, cp)
-    key = (ws2.device.index or 0, ws2.data_ptr(), cp)
+    key = (ws2.data_ptr(), cp)
     assert key in ops._groups
     torch.cuda.synchronize()
+    # ... and keeps that workspace alive while ranks are waiting, whatever the caller does with its handle
     del ws2
     import gc
     gc.collect()
-    assert key not in ops._groups
+    assert ops._groups[key].pending and ops._groups[key].workspace is not None
+    ops.reset_logical_ranks()
+    assert not ops._groups
 
 
 @pytest.mark.parametrize("single_round", [False, True])
@@ -899,7 +963,7 @@ def test_receivers_overlapping_their_senders(hx, ops, channels):
     # With few channels every wavefront of the launch is resident at once and receivers poll FIFO
     # lines while their senders are still writing them. A receiver that consumed a line on the
     # strength of a flag it had read in the same pass as the payload could see a half-written line.
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS["c3"]
     ws = get_workspace(hx, w.cp)
@@ -927,7 +991,7 @@ def test_exchange_and_combine_replay_from_a_captured_graph(hx, ops):
     # The FIFO step counters live in the workspace, not in the kernel arguments, so a captured
     # launch can be replayed: every replay walks on to the next FIFO entry. Replays are interleaved
     # with eager work and synchronisations, and every one of them is checked.
-    from helix_a2a.workloads import WORKLOADS, make_inputs
+    from helix_workloads import WORKLOADS, make_inputs
 
     w = WORKLOADS["c2"]
     ws = get_workspace(hx, w.cp)
@@ -1041,7 +1105,7 @@ def test_empty_inputs(hx, ops):
     check_against_oracle(o1, s1, got_o, got_s)
 
 
-def test_per_rank_calls_on_separate_streams(hx, ops):
+def test_per_rank_calls_on_separate_streams(hx, ops, send_policy):
     # every logical rank calls on a stream of its own and waits for that stream only
     cp, entries = 4, 96
     ws = get_workspace(hx, cp)
@@ -1064,7 +1128,7 @@ def test_per_rank_calls_on_separate_streams(hx, ops):
     assert_clean(ops)
 
 
-def test_per_rank_calls_replay_from_a_captured_graph(hx, ops):
+def test_per_rank_calls_replay_from_a_captured_graph(hx, ops, send_policy):
     # the reference's signature, one call per logical rank, captured once and replayed on fresh payload
     cp, entries = 4, 64
     ws = get_workspace(hx, cp)
@@ -1096,7 +1160,7 @@ def test_per_rank_calls_replay_from_a_captured_graph(hx, ops):
     assert_clean(ops)
 
 
-def test_reference_environment_switches(hx, ops, monkeypatch):
+def test_reference_environment_switches(hx, ops, monkeypatch, send_policy):
     # HELIX_A2A_ENABLE_PDL (csrc/helix_alltoall.cu:541-548) is accepted and changes nothing: ordering between
     # calls is stream order. HELIX_A2A_CHANNEL_COUNT (csrc/torch_binding.cpp:25-32) is honoured, re-read per call.
     cp = 4
