@@ -311,6 +311,122 @@ def memory_probe(mib: int = 1024, reps: int = 20):
     return out
 
 
+PROBE_LIB = ROOT / "helix-a2a_amd" / "benchmark" / "libhelix_memory_probe.so"
+
+
+def exchange_kernel_timing(w, steps: int = 200, warmup: int = 30):
+    """Event-timed exchange launches of one workload, hot (one set of tensors) and cold (rotating sets, 1 GiB)."""
+    import torch
+
+    import helix_a2a
+    from helix_a2a import _ops
+    from helix_workloads import make_inputs
+
+    ws = helix_a2a.allocate_workspace(w.cp, 0)
+    for r in range(w.cp):
+        helix_a2a.init_workspace(ws, r, w.cp)
+    ins_o, ins_s = make_inputs(w, "cuda")
+    channels = _ops.auto_channel_count(w.cp, w.tokens)
+    nbytes = w.exchange_bytes(channels)
+    tensor_bytes = sum(t.numel() * t.element_size() for t in ins_o + ins_s) * 2
+    n_sets = max(2, -(-(1 << 30) // tensor_bytes))
+    plans = [_ops.LoopbackPlan(ins_o, ins_s, ws)]
+    hot = _event_us(plans[0].run, steps, warmup)
+    plans += [_ops.LoopbackPlan([t.clone() for t in ins_o], [t.clone() for t in ins_s], ws) for _ in range(n_sets - 1)]
+    turn = [0]
+
+    def next_set():
+        plans[turn[0] % n_sets].run()
+        turn[0] += 1
+
+    cold = _event_us(next_set, steps, max(warmup, n_sets))
+    status = _ops.device_status()
+    del plans, ws
+    torch.cuda.empty_cache()
+    return {"channels": channels, "algorithmic_bytes_per_call": nbytes, "kernel_us": hot, "kernel_us_cold": cold,
+            "frac": nbytes / (hot * 1e-6) / 1e9 / PEAK_HBM_GBPS, "frac_cold": nbytes / (cold * 1e-6) / 1e9 / PEAK_HBM_GBPS,
+            "status": status}
+
+
+def chunk_copy_probe(names=("c3", "c4", "c5a"), reps: int = 40, kernel_us=None):
+    """What a plain chunked copy of each workload's shape reaches on this box (helix-a2a_amd/benchmark/memory_probe.hip):
+    one chunk per stream, as long as the stream's run of LL128 lines, moved by as many wavefronts as the exchange
+    kernel gives a run, in the same passes of 16-byte units -- no counters, tokens, flags or index arithmetic.
+    `send`: dense memory -> FIFO-like slots 512 KiB apart (the entry of a slot rotating through its four positions,
+    as the FIFOs' do); `recv`: slots -> dense. Hot re-uses one dense buffer per side, cold takes the next of N
+    (1 GiB in rotation). `copy_bound_us` = send + recv, each scaled from the probe's bytes (lines in, lines out) to
+    the exchange's (payload + lines): the time the two halves of the exchange would take at the probe's rates.
+    `kernel_us`: {workload: (hot, cold)} of the exchange kernel, to put beside it."""
+    import ctypes
+
+    import torch
+
+    from helix_a2a import _ops
+    from helix_workloads import WORKLOADS
+
+    if not PROBE_LIB.exists():
+        return {"error": f"{PROBE_LIB.name} not built (python helix-a2a_amd/build.py --probe)"}
+    lib = ctypes.CDLL(str(PROBE_LIB))
+    lib.helix_probe_chunk_copy.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_uint64,
+                                           ctypes.c_uint32, ctypes.c_uint32, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.helix_probe_chunk_copy.restype = ctypes.c_int
+    slot, entry = 512 * 1024, 128 * 1024
+    out = {}
+    for name in names:
+        w = WORKLOADS[name]
+        channels = _ops.auto_channel_count(w.cp, w.tokens)
+        streams = w.cp * w.cp * channels
+        wire = w.run_wire_bytes(channels)
+        if w.tokens % channels or wire % streams:
+            out[name] = {"error": "streams of unequal runs"}
+            continue
+        runs_per_stream = -(-(w.tokens // channels) // (1024 * 15 // ((w.field0_bytes + w.field1_bytes) // 8)))
+        chunk = wire // streams // runs_per_stream
+        per_lane = -(-chunk // 1024)
+        passes = -(-per_lane // 6)
+        team = min(passes, 8) if passes >= 3 and 2 * streams > 4096 else 1   # the exchange kernel's rule for teams
+        dense_bytes = streams * chunk
+        n_sets = max(2, -(-(1 << 30) // (2 * dense_bytes)))
+        slots = torch.empty(streams * slot, dtype=torch.uint8, device="cuda")
+        slots.fill_(1)
+        dense = [torch.full((dense_bytes,), 2, dtype=torch.uint8, device="cuda") for _ in range(2 * n_sets)]
+        stream = _ops._stream_handle()
+        turn = [0]
+
+        def leg(send: bool, cold: bool):
+            i = turn[0]
+            turn[0] += 1
+            d = dense[(2 * (i % n_sets) if cold else 0) + (0 if send else 1)]
+            s_ptr = slots.data_ptr() + (i % 4) * entry
+            if send:
+                rc = lib.helix_probe_chunk_copy(d.data_ptr(), chunk, s_ptr, slot, chunk, streams, team, 0, stream)
+            else:
+                rc = lib.helix_probe_chunk_copy(s_ptr, slot, d.data_ptr(), chunk, chunk, streams, team, 0, stream)
+            if rc != 0:
+                raise RuntimeError(f"helix_probe_chunk_copy failed: {rc}")
+
+        row = {"chunk_bytes": chunk, "chunks": streams, "wavefronts_per_chunk": team}
+        scale = (w.payload_bytes / runs_per_stream + wire / runs_per_stream) / (2.0 * dense_bytes)  # exchange half / probe leg, in bytes
+        for cold in (False, True):
+            tag = "cold" if cold else "hot"
+            send_us = _event_us(lambda: leg(True, cold), reps, 2 * n_sets if cold else 5)
+            recv_us = _event_us(lambda: leg(False, cold), reps, 2 * n_sets if cold else 5)
+            row[tag] = {"send_us": send_us, "recv_us": recv_us,
+                        "send_GBps": 2 * dense_bytes / send_us / 1e3, "recv_GBps": 2 * dense_bytes / recv_us / 1e3,
+                        "copy_bound_us": (send_us + recv_us) * scale * runs_per_stream}
+            if kernel_us and name in kernel_us:
+                k = kernel_us[name][1 if cold else 0]
+                if k:
+                    row[tag]["exchange_kernel_us"] = k
+                    row[tag]["exchange_over_copy_bound"] = k / row[tag]["copy_bound_us"]
+        out[name] = row
+        del slots, dense
+        torch.cuda.empty_cache()
+    out["note"] = ("plain chunked copies of each workload's shape (one chunk per stream, its run of lines; dense <-> slots "
+                   "512 KiB apart), GB/s of bytes read + written; copy_bound_us = the two halves of the exchange at these rates")
+    return out
+
+
 def cold_only(args, w, make_plan, ins_o, ins_s, bytes_per_call) -> int:
     """The cold leg alone: every step on the next of N sets of tensors; prints a short JSON line."""
     import torch
@@ -363,6 +479,9 @@ def main() -> int:
     ap.add_argument("--team-units", type=int, default=None, metavar="U",
                     help="teams of wavefronts per stream: 1..6 always (at most U KiB per wavefront), 0 never, "
                          "-1 the library's rule (runs of three or more passes in launches that queue)")
+    ap.add_argument("--probe", choices=("chunk-copy",), default=None,
+                    help="chunk-copy: print only the memory probe -- plain chunked copies of the shapes of c3, c4 and c5a, "
+                         "hot and cold, beside the exchange kernel on the same workloads -- as one JSON line")
     ap.add_argument("--no-host-timing", action="store_true", help="skip the host-time-per-call measurements")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
@@ -385,6 +504,11 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
     torch.cuda.set_device(0)
+    if args.probe == "chunk-copy":
+        timings = {n: exchange_kernel_timing(WORKLOADS[n], max(args.steps, MIN_ROOFLINE_STEPS)) for n in ("c3", "c4", "c5a")}
+        probe = chunk_copy_probe(kernel_us={n: (t["kernel_us"], t["kernel_us_cold"]) for n, t in timings.items()})
+        print(json.dumps({"probe": "chunk-copy", "exchange": timings, "chunk_copy": probe, "plain": memory_probe()}))
+        return 0 if all(t["status"] == 0 for t in timings.values()) else 1
     w = WORKLOADS[args.workload]
     ws = helix_a2a.allocate_workspace(w.cp, 0)
     for r in range(w.cp):
@@ -591,6 +715,14 @@ def main() -> int:
         del plan
         result["per_rank_gpu_us"] = per_rank_gpu_timing(spare=(w.name, ws))
         result["decode_sizes_us"] = decode_size_timing()
+        # the workloads beyond the memory-side cache, and what a plain chunked copy of each shape reaches in this run
+        del ws, ins_o, ins_s
+        torch.cuda.empty_cache()
+        others = {n: exchange_kernel_timing(WORKLOADS[n]) for n in ("c4", "c5a") if n != w.name}
+        result["other_workloads"] = others
+        kernel_us = {n: (t["kernel_us"], t["kernel_us_cold"]) for n, t in others.items()}
+        kernel_us[w.name] = (avg_kernel_ms * 1e3, cold["kernel_us"] if cold else None)
+        result["memory_probe"]["chunk_copy"] = chunk_copy_probe(kernel_us=kernel_us)
     if not args.no_cpu_baseline and not args.combine and args.layout == "token":
         result["cpu_baseline"] = cpu_baseline(w, bytes_per_call)
     print(json.dumps(result))

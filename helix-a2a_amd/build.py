@@ -57,7 +57,25 @@ def build_library(verbose: bool = True, timeline: bool = False) -> Path:
     return output
 
 
+PROBE_SOURCE = HERE / "benchmark" / "memory_probe.hip"
+PROBE_OUTPUT = HERE / "benchmark" / "libhelix_memory_probe.so"
+
+
+def build_memory_probe(verbose: bool = True) -> Path:
+    """The chunked-copy yardstick of bench.py --probe chunk-copy (measuring equipment, a library of its own)."""
+    cmd = [find_hipcc(), *HIPCC_FLAGS, str(PROBE_SOURCE), "-o", str(PROBE_OUTPUT)]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed with exit code {proc.returncode}\n{proc.stdout}{proc.stderr}")
+    return PROBE_OUTPUT
+
+
 if __name__ == "__main__":
-    out = build_library(timeline="--timeline" in sys.argv[1:])
+    if "--probe" in sys.argv[1:]:
+        out = build_memory_probe()
+    else:
+        out = build_library(timeline="--timeline" in sys.argv[1:])
     print(f"built {out}")
     sys.exit(0)

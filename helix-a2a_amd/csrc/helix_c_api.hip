@@ -289,6 +289,10 @@ int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs,
                   static_cast<unsigned long long>(workspace_bytes(cp, maxCh)), cp);
   }
 
+  // a wavefront's descriptor of its stream's lines reaches over three quarters of the FIFO region and a slot
+  if (static_cast<uint64_t>(kFifoDepth - 1) * fifo_position_bytes(cp, maxCh) + kFifoEntryBytes >= 0x80000000ull)
+    return fail(HELIX_A2A_ERR_INVALID_ARGUMENT, "a FIFO region of %d x %d streams is beyond what the kernels address", cp, maxCh);
+
   int channels = p0.channel_count > 0 ? p0.channel_count : env_channel_count();
   if (channels > maxCh) {
     if (p0.channel_count > 0 || builtin == nullptr)

@@ -42,7 +42,8 @@
 // before its first store.
 //
 // Every global access goes through a buffer descriptor that spans exactly the
-// tensor (or the one FIFO) it belongs to: the hardware returns zero for loads
+// tensor it belongs to (for FIFO lines: the stream's slots, first quarter of
+// the FIFO region to last): the hardware returns zero for loads
 // and drops stores that would fall outside, and an offset of kOutOfRange is
 // how a lane opts out of an access without a branch.
 //
@@ -156,6 +157,10 @@ __device__ __forceinline__ uint64_t* broken_word(const KernelArgs& a) {
   return reinterpret_cast<uint64_t*>(a.workspace + broken_word_offset(a.cpSize, a.maxChannels));
 }
 
+// How far a wavefront's descriptor of its stream's lines reaches: from the stream's slot in the first quarter of
+// the FIFO region to the end of its slot in the last one (the entry of a step sits in quarter step & 3).
+__device__ __forceinline__ uint32_t fifo_extent(const KernelArgs& a) { return (kFifoDepth - 1) * a.positionBytes + a.slotBytes; }
+
 // Whether the workspace was broken before this launch started. A wave-uniform read through the scalar
 // cache (which starts every launch empty): it costs no vector memory instruction, and it need not see
 // what the running launch does to the word -- the bounded waits look at that themselves.
@@ -212,7 +217,7 @@ __device__ __forceinline__ void fetch_scalars_up_front(const KernelArgs& a) {
   asm volatile("" ::"s"(a.parts), "s"(a.team), "s"(a.np0), "s"(a.np), "s"(a.msgsPerEntry), "s"(a.baseMsgs),
                "s"(a.extraChannels), "s"(a.byParts.magic), "s"(a.byParts.shift), "s"(a.byTeam.magic), "s"(a.byTeam.shift),
                "s"(a.byCp.magic), "s"(a.byCp.shift), "s"(a.byChannels.magic), "s"(a.byChannels.shift), "s"(a.sendBlocks), "s"(a.wavesPerBlock), "s"(a.dirBlocks), "s"(a.xcdGroup),
-               "s"(a.spinLimitTicks));
+               "s"(a.spinLimitTicks), "s"(a.slotBytes), "s"(a.positionBytes));
 }
 
 // What a stream's wavefront needs to know, all wave-uniform.
@@ -290,7 +295,7 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
   uint8_t* receiverRow = a.workspace + static_cast<uint64_t>(r) * a.rowStrideBytes;
   int64_t* info = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(a.cpSize, a.maxChannels, r, ch));
   int64_t* token = info + sender_counter_slot(kTeam ? 0 : part);
-  st.fifo = make_rsrc(receiverRow + fifo_offset(s, ch, a.maxChannels), kFifoBytes);
+  st.fifo = make_rsrc(receiverRow + stream_fifo_offset(s, ch, a.runChannels, a.slotBytes), fifo_extent(a));
   st.field0 = make_rsrc(a.rank[s].send0, a.sendBytes0);
   st.field1 = make_rsrc(a.rank[s].send1, a.sendBytes1);
   st.stride0 = a.sendStride0;
@@ -390,7 +395,7 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
       }
       if (!opened && !open_entry()) return;
       if (U0 == slice.begin && firstMsg == 0) HELIX_MARK(wave, 1, true);
-      const uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
+      const uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * a.positionBytes;
       const uint32_t stepLo = static_cast<uint32_t>(step);
       const uint32_t stepHi = static_cast<uint32_t>(static_cast<uint64_t>(step) >> 32);
 #pragma unroll
@@ -436,7 +441,7 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
   int64_t* info = reinterpret_cast<int64_t*>(receiverRow + receiver_info_offset(a.cpSize, a.maxChannels, s, ch));
   int64_t* token = senderInfo + sender_counter_slot(counterPart);
   int64_t* mine = info + receiver_counter_slot(counterPart);
-  st.fifo = make_rsrc(receiverRow + fifo_offset(s, ch, a.maxChannels), kFifoBytes);
+  st.fifo = make_rsrc(receiverRow + stream_fifo_offset(s, ch, a.runChannels, a.slotBytes), fifo_extent(a));
   st.field0 = make_rsrc(a.rank[r].recv0, a.recvBytes0);
   st.field1 = make_rsrc(a.rank[r].recv1, a.recvBytes1);
   st.stride0 = a.recvStride0;
@@ -495,7 +500,7 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
       if (step < 0) return;
     }
     asm volatile("" ::: "memory");  // no line is read before the token was seen
-    const uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
+    const uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * a.positionBytes;
     const uint32_t stepLo = static_cast<uint32_t>(step);
     const uint32_t stepHi = static_cast<uint32_t>(static_cast<uint64_t>(step) >> 32);
     for (uint32_t U0 = slice.begin; U0 < slice.end; U0 += kUnitsInFlight * kWaveLanes) {
@@ -688,6 +693,7 @@ struct CombineCtx {
   uint32_t channelBase;          // byte offset of sender 0's FIFO of this channel
   uint32_t senderStride;         // bytes between the FIFOs of consecutive senders
   uint32_t stepLo;               // lane q: step counter (low word) of sender q's stream
+  uint32_t positionBytes;        // bytes between the four positions an entry of a stream rotates through
 };
 
 template <int kLanesPerSlot>
@@ -700,7 +706,7 @@ __device__ __forceinline__ float shuffle_xor(float v, int mask) { return __shfl_
 
 // byte offset of sender q's open FIFO entry inside the receiver's FIFO region
 __device__ __forceinline__ uint32_t entry_base(const CombineCtx& cx, int q, uint32_t stepLo) {
-  return cx.channelBase + static_cast<uint32_t>(q) * cx.senderStride + (stepLo & (kFifoDepth - 1)) * kFifoEntryBytes;
+  return cx.channelBase + static_cast<uint32_t>(q) * cx.senderStride + (stepLo & (kFifoDepth - 1)) * cx.positionBytes;
 }
 
 // byte offset of run piece g inside a FIFO entry: line g / 15, word g % 15
@@ -763,8 +769,9 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
   uint8_t* receiverRow = a.workspace + static_cast<uint64_t>(r) * a.rowStrideBytes;
   CombineCtx cx;
   cx.fifos = make_rsrc(receiverRow, static_cast<uint32_t>(fifo_region_bytes(a.cpSize, a.maxChannels)));
-  cx.channelBase = static_cast<uint32_t>(fifo_offset(0, ch, a.maxChannels));
-  cx.senderStride = static_cast<uint32_t>(fifo_offset(1, 0, a.maxChannels));
+  cx.channelBase = static_cast<uint32_t>(stream_fifo_offset(0, ch, a.runChannels, a.slotBytes));
+  cx.senderStride = static_cast<uint32_t>(stream_fifo_offset(1, 0, a.runChannels, a.slotBytes));
+  cx.positionBytes = a.positionBytes;
   __amdgpu_buffer_rsrc_t outRsrc = make_rsrc(a.rank[r].recv0, a.recvBytes0);
   __amdgpu_buffer_rsrc_t lseRsrc = make_rsrc(a.rank[r].recv1, a.rank[r].recv1 ? a.recvBytes1 : 0u);
   const unsigned long long lanesUpToMe = (2ull << lane) - 1ull;  // lanes 0..lane
@@ -1035,6 +1042,8 @@ static void set_launch_constants(KernelArgs& a) {
   a.extraChannels = entries % a.runChannels;
   a.entriesBase = entries_for_msgs(a.baseMsgs, sh);
   a.entriesExtra = entries_for_msgs(a.baseMsgs + 1, sh);
+  a.slotBytes = packed_slot_bytes(largest_run_units(a));
+  a.positionBytes = fifo_position_bytes(a.cpSize, a.maxChannels);
   a.byParts = fast_div(static_cast<uint32_t>(a.parts));
   a.byTeam = fast_div(static_cast<uint32_t>(a.team));
   a.byCp = fast_div(static_cast<uint32_t>(a.cpSize));

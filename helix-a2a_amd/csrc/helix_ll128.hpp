@@ -22,17 +22,25 @@
 // line boundaries fall (a 264-byte message is 33 pieces = 2.2 lines, not 3).
 // Only the last line of a run is zero padded.
 //
-// Workspace geometry (one row per rank, unchanged from the reference so that
-// workspace_size and the init pattern stay drop-in,
-// csrc/helix_alltoall.cu:61-75,194-242,605-614):
+// Workspace geometry (one row per rank; the regions, their sizes and the init
+// pattern are the reference's, so that workspace_size and init_workspace stay
+// drop-in, csrc/helix_alltoall.cu:61-75,194-242,605-614):
 //
 //   [ FIFO region : cp senders x maxCh channels x 4 entries x 128 KiB ]
 //   [ sender info : cp receivers x maxCh x 256 B  {int64 head; int64 tail} ]
 //   [ receiver info: cp senders  x maxCh x 256 B  {int64 head; int64 tail} ]
 //
-//   FIFO of (sender s -> receiver r, channel c) lives in row r at
-//   (s*maxCh + c) * 512 KiB; the sender's counters live in row s indexed by r,
-//   the receiver's counters in row r indexed by s.
+//   The sender's counters of stream (s -> r, channel c) live in row s indexed by
+//   r, the receiver's counters in row r indexed by s, as in the reference.
+//   Where the stream's lines live inside row r's FIFO region is this build's
+//   own (nothing outside the kernels reads them): the region is four quarters,
+//   one per position a stream's entry rotates through (step & 3), and inside a
+//   quarter a launch packs its streams side by side, a slot of
+//   packed_slot_bytes(largest run of the launch) each -- see stream_fifo_offset.
+//   (The reference gives every stream four 128 KiB entries of its own,
+//   512 KiB apart: a launch's lines are then spread thinly over the whole
+//   region, which measured 3-9 % slower on MI355X wherever runs are long or a
+//   wavefront reads the lines of many senders.)
 #pragma once
 
 #include <stdint.h>
@@ -87,9 +95,26 @@ HELIX_HD uint64_t workspace_bytes(int cpSize, int maxCh) {
   return fifo_region_bytes(cpSize, maxCh) + 2 * info_region_bytes(cpSize, maxCh);
 }
 
-// byte offset inside the RECEIVER's row (csrc/helix_alltoall.cu:194-206)
-HELIX_HD uint64_t fifo_offset(int sender, int channel, int maxCh) {
-  return (static_cast<uint64_t>(sender) * maxCh + channel) * kFifoBytes;
+// ---- where a launch puts its runs inside the receiver row's FIFO region ----------
+// A stream's entry of step k sits in quarter k & 3 of the region; a quarter is cp * maxCh * 128 KiB, room for a
+// full 128 KiB entry of every stream the layout provides for. Within the quarter the streams of a launch are
+// packed: stream (sender, channel) of a launch over runChannels channels starts at
+// (sender * runChannels + channel) * slotBytes, and slotBytes is the launch's largest run (every launch knows it:
+// channel 0's first run) rounded up to whole KiB -- but runs shorter than 8 KiB are kept 16 KiB apart (4.5 KiB
+// runs packed closer than that measured 2-16 % slower). Sender and receiver of a launch derive the same
+// slotBytes from the same launch shape; between launches nothing but the counters is carried over, so launches
+// of different shapes may place their lines differently.
+HELIX_HD uint32_t fifo_position_bytes(int cpSize, int maxCh) {
+  return static_cast<uint32_t>(static_cast<uint64_t>(kFifoEntryBytes) * cpSize * maxCh);  // a quarter of the region, < 2^32
+}
+HELIX_HD uint32_t packed_slot_bytes(long largestRunUnits) {
+  const long bytes = largestRunUnits * kUnitBytes;
+  if (bytes < 8192) return 16384;
+  return static_cast<uint32_t>((bytes + 1023) / 1024 * 1024);  // at most kFifoEntryBytes: a run is at most 1024 lines
+}
+// byte offset of the stream's slot inside a quarter of the RECEIVER's row
+HELIX_HD uint64_t stream_fifo_offset(int sender, int channel, int runChannels, uint32_t slotBytes) {
+  return (static_cast<uint64_t>(sender) * runChannels + channel) * slotBytes;
 }
 // byte offset inside the SENDER's row (csrc/helix_alltoall.cu:208-223)
 HELIX_HD uint64_t sender_info_offset(int cpSize, int maxCh, int receiver, int channel) {

@@ -65,9 +65,11 @@ class HostModel:
         lib.hm_alltoall.argtypes = [ctypes.POINTER(_Params)] + [ctypes.c_int] * 5
         lib.hm_alltoall.restype = ctypes.c_int
         lib.hm_last_message.restype = ctypes.c_char_p
-        for name in ("hm_fifo_offset",):
-            getattr(lib, name).argtypes = [ctypes.c_int] * 3
-            getattr(lib, name).restype = ctypes.c_uint64
+        lib.hm_stream_fifo_offset.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_long, ctypes.c_int,
+                                              ctypes.c_int, ctypes.c_long]
+        lib.hm_stream_fifo_offset.restype = ctypes.c_uint64
+        lib.hm_packed_slot_bytes.argtypes = [ctypes.c_long]
+        lib.hm_packed_slot_bytes.restype = ctypes.c_uint32
         for name in ("hm_sender_info_offset", "hm_receiver_info_offset"):
             getattr(lib, name).argtypes = [ctypes.c_int] * 4
             getattr(lib, name).restype = ctypes.c_uint64
@@ -96,6 +98,13 @@ class HostModel:
         lib.hm_msgs_per_entry.argtypes = [ctypes.c_int] * 2
         lib.hm_msgs_per_entry.restype = ctypes.c_int
         self.lib = lib
+
+    def stream_fifo_offset(self, sender: int, channel: int, run_channels: int, largest_run_lines: int, cp: int,
+                           cu_count: int, step: int = 0) -> int:
+        """Byte offset inside the receiver's row of the lines stream (sender, channel) writes under ``step`` in a launch
+        over ``run_channels`` channels whose largest run has ``largest_run_lines`` lines."""
+        return self.lib.hm_stream_fifo_offset(sender, channel, run_channels, largest_run_lines * 8, cp,
+                                              self.max_channel_count(cp, cu_count), step)
 
     def split_for_run(self, run_units: int, units_per_part: int = 6, max_parts: int = 16) -> Tuple[int, int]:
         """(wavefronts per stream, units in flight) the launch rule picks for a largest run of ``run_units`` units."""

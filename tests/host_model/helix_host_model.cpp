@@ -51,6 +51,12 @@ struct Ctx {
   int unitsInFlight;   // per round, by the library's rule
   int parts;           // wavefronts that share a stream's runs, by the library's rule
   bool alignedStores;  // receivers of long runs store realigned 16-byte pieces
+  uint32_t slotBytes, positionBytes;  // where the round's streams put their lines (packed_slot_bytes, fifo_position_bytes)
+  // the FIFO region of rank r's row
+  Extent fifoRegion(int r) const {
+    return Extent{reinterpret_cast<const uint8_t*>(ranks[0].workspace) + r * ranks[0].workspace_stride_u64 * 8,
+                  fifo_region_bytes(cp, maxCh)};
+  }
 };
 
 int g_unitsPerPart = -1;  // the library's knob: -1 automatic, 0 one wavefront per stream, 1..6 share runs longer than that per lane
@@ -93,10 +99,9 @@ void run_sender(Ctx& c, int s, int r, int ch, int part) {
   uint8_t* senderRow = wsBase + s * rowStride;
   uint8_t* receiverRow = wsBase + r * rowStride;
   int64_t* info = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(c.cp, c.maxCh, r, ch));
-  uint8_t* fifo = receiverRow + fifo_offset(s, ch, c.maxCh);
-  if (!c.chk.ok(c.ws, info, kFifoInfoBytes, "sender info") || !c.chk.ok(c.ws, fifo, kFifoBytes, "fifo")) return;
+  uint8_t* fifo = receiverRow + stream_fifo_offset(s, ch, c.channels, c.slotBytes);
+  if (!c.chk.ok(c.ws, info, kFifoInfoBytes, "sender info")) return;
   int64_t* token = info + sender_counter_slot(part);
-  Extent fifoExt{fifo, kFifoBytes};
   Extent e0 = field_extent(p.send_fields[0], p.entry_count, c.cp);
   Extent e1 = field_extent(p.send_fields[1], p.entry_count, c.cp);
   const int msgs = stream_msg_count(c.entryBegin, c.entryEnd, ch, c.channels);
@@ -120,7 +125,10 @@ void run_sender(Ctx& c, int s, int r, int ch, int part) {
                (long long)step);
       return;
     }
-    uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
+    uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * c.positionBytes;
+    // tighter than the GPU's descriptor: every access must stay inside the stream's slot of this step's quarter
+    Extent fifoExt{fifo + entryOffset, c.slotBytes};
+    if (!c.chk.ok(c.fifoRegion(r), fifoExt.base, c.slotBytes, "fifo slot")) return;
     for (uint32_t U = slice.begin; U < slice.end; ++U) {  // every lane of every wave access
       UnitOffsets o = unit_offsets(c, firstRow, rowStep, p.send_fields[0].stride_bytes, p.send_fields[1].stride_bytes,
                                    firstMsg, runMsgs, U);
@@ -148,13 +156,10 @@ void run_receiver(Ctx& c, int r, int s, int ch, int part) {
   uint8_t* receiverRow = wsBase + r * rowStride;
   int64_t* sinfo = reinterpret_cast<int64_t*>(senderRow + sender_info_offset(c.cp, c.maxCh, r, ch));
   int64_t* info = reinterpret_cast<int64_t*>(receiverRow + receiver_info_offset(c.cp, c.maxCh, s, ch));
-  uint8_t* fifo = receiverRow + fifo_offset(s, ch, c.maxCh);
-  if (!c.chk.ok(c.ws, info, kFifoInfoBytes, "receiver info") || !c.chk.ok(c.ws, sinfo, kFifoInfoBytes, "sender info") ||
-      !c.chk.ok(c.ws, fifo, kFifoBytes, "fifo"))
-    return;
+  uint8_t* fifo = receiverRow + stream_fifo_offset(s, ch, c.channels, c.slotBytes);
+  if (!c.chk.ok(c.ws, info, kFifoInfoBytes, "receiver info") || !c.chk.ok(c.ws, sinfo, kFifoInfoBytes, "sender info")) return;
   const int64_t* token = sinfo + sender_counter_slot(part);
   int64_t* mine = info + receiver_counter_slot(part);
-  Extent fifoExt{fifo, kFifoBytes};
   Extent e0 = field_extent(p.recv_fields[0], p.entry_count, c.cp);
   Extent e1 = field_extent(p.recv_fields[1], p.entry_count, c.cp);
   const int msgs = stream_msg_count(c.entryBegin, c.entryEnd, ch, c.channels);
@@ -178,7 +183,9 @@ void run_receiver(Ctx& c, int r, int s, int ch, int part) {
                  part, (long long)*token, (long long)step);
       return;
     }
-    uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * kFifoEntryBytes;
+    uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * c.positionBytes;
+    Extent fifoExt{fifo + entryOffset, c.slotBytes};
+    if (!c.chk.ok(c.fifoRegion(r), fifoExt.base, c.slotBytes, "fifo slot")) return;
     uint8_t* base0 = const_cast<uint8_t*>(e0.base);
     uint8_t* base1 = const_cast<uint8_t*>(e1.base);
     const uint32_t stride0 = p.recv_fields[0].stride_bytes, stride1 = p.recv_fields[1].stride_bytes;
@@ -308,6 +315,8 @@ int hm_alltoall(const helix_a2a_params_t* per_rank, int cp, int cu_count, int ch
       c.parts = split.parts;
       c.unitsInFlight = split.unitsInFlight;
       c.alignedStores = maxRun > static_cast<long>(kMaxUnitsInFlight) * kWaveLanes;
+      c.slotBytes = packed_slot_bytes(maxRun);
+      c.positionBytes = fifo_position_bytes(cp, c.maxCh);
     }
     if (c.parts > 1) level_part_counters(c, do_send != 0, do_recv != 0);
     if (do_send)
@@ -335,7 +344,13 @@ int hm_split_for_run(long runUnits, int unitsPerPart, int maxParts) {
 }
 
 // geometry probes for tests
-uint64_t hm_fifo_offset(int sender, int channel, int max_ch) { return fifo_offset(sender, channel, max_ch); }
+// byte offset, inside the receiver's row, of the lines stream (sender, channel) writes under step `step` in a launch
+// over `run_channels` channels whose largest run has `largest_run_units` units
+uint64_t hm_stream_fifo_offset(int sender, int channel, int run_channels, long largest_run_units, int cp, int max_ch, long step) {
+  return stream_fifo_offset(sender, channel, run_channels, packed_slot_bytes(largest_run_units)) +
+         static_cast<uint64_t>(step & (kFifoDepth - 1)) * fifo_position_bytes(cp, max_ch);
+}
+uint32_t hm_packed_slot_bytes(long largest_run_units) { return packed_slot_bytes(largest_run_units); }
 uint64_t hm_sender_info_offset(int cp, int max_ch, int receiver, int channel) {
   return sender_info_offset(cp, max_ch, receiver, channel);
 }

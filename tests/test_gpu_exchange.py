@@ -626,10 +626,8 @@ def test_fifo_image_matches_host_model(hx, ops, host_model):
     max_ch = host_model.max_channel_count(cp, cu)
     fifo_region_elems = FIFO_BYTES * cp * max_ch // 8
     for row in range(cp):
-        for sender in range(cp):
-            off = host_model.lib.hm_fifo_offset(sender, 0, max_ch) // 8
-            got = ws[row, off: off + FIFO_BYTES // 8].cpu().numpy()
-            assert np.array_equal(got, host_ws[row, off: off + FIFO_BYTES // 8]), f"FIFO {sender}->{row} differs"
+        # the whole FIFO region: the lines of every stream where the launch packed them, 0xFF everywhere else
+        assert np.array_equal(ws[row, :fifo_region_elems].cpu().numpy(), host_ws[row, :fifo_region_elems]), f"FIFO region of row {row} differs"
         assert np.array_equal(ws[row, fifo_region_elems:].cpu().numpy(), host_ws[row, fifo_region_elems:])
     # finish the exchange so the workspace is consistent again
     ops._check(ops._lib.helix_a2a_alltoall_recv(arr, cp, ops._stream_handle()), "recv")

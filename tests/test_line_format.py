@@ -72,21 +72,24 @@ def test_line_layout_in_fifo(host_model):
     assert rc == 0, msg
     max_ch = host_model.max_channel_count(cp, CU)
     assert host_model.lib.hm_msg_lines(2 * x, 4 * s) == 9
-    for sender in range(cp):
-        for receiver in range(cp):
-            off = host_model.lib.hm_fifo_offset(sender, 0, max_ch)
-            assert off == (sender * max_ch) * FIFO_BYTES
-            fifo = ws[receiver].view(np.uint64)[off // 8: (off + FIFO_BYTES) // 8]
-            lines = fifo[: 9 * 16].reshape(9, 16)
+    fifo_region = FIFO_BYTES * cp * max_ch
+    for receiver in range(cp):
+        region = ws[receiver].view(np.uint64)[: fifo_region // 8]
+        untouched = np.ones(region.size, dtype=bool)
+        for sender in range(cp):
+            # a launch packs its streams: runs shorter than 8 KiB sit 16 KiB apart, in the quarter of step & 3
+            off = host_model.stream_fifo_offset(sender, 0, 1, 9, cp, CU)
+            assert off == sender * 16384
+            lines = region[off // 8: off // 8 + 9 * 16].reshape(9, 16)
+            untouched[off // 8: off // 8 + 9 * 16] = False
             payload = np.concatenate([ins_o[sender][0, receiver].view(np.uint64), ins_s[sender][0, receiver].view(np.uint64)])
             assert payload.size == 132
             padded = np.zeros(9 * 15, dtype=np.uint64)
             padded[:132] = payload
             assert (lines[:, :15] == padded.reshape(9, 15)).all()   # 15 payload words per line, in order
             assert (lines[:, 15] == 0).all()                        # flag word = step 0 of a fresh workspace
-            assert (fifo[9 * 16:] == np.uint64(0xFFFFFFFFFFFFFFFF)).all()  # nothing else was touched
+        assert (region[untouched] == np.uint64(0xFFFFFFFFFFFFFFFF)).all()  # nothing else was touched
     # counters: each sender stream consumed one FIFO entry; the receiver has not run
-    fifo_region = FIFO_BYTES * cp * max_ch
     for sender in range(cp):
         for receiver in range(cp):
             so = host_model.lib.hm_sender_info_offset(cp, max_ch, receiver, 0)
@@ -96,6 +99,34 @@ def test_line_layout_in_fifo(host_model):
             ro = host_model.lib.hm_receiver_info_offset(cp, max_ch, sender, 0)
             assert ro == fifo_region + INFO_BYTES * cp * max_ch + (sender * max_ch) * INFO_BYTES
             assert ws[receiver][ro // 8 + 1] == 0
+
+
+def test_packed_layout_keeps_the_streams_of_a_launch_apart(host_model):
+    # a launch packs its streams inside a quarter of the FIFO region: every slot holds the largest run, no two
+    # streams overlap, everything stays inside the quarter, and the four positions are a quarter apart
+    assert host_model.lib.hm_packed_slot_bytes(8) == 16384                 # one line
+    assert host_model.lib.hm_packed_slot_bytes(36 * 8) == 16384            # 4.5 KiB: short runs sit 16 KiB apart
+    assert host_model.lib.hm_packed_slot_bytes(63 * 8) == 16384
+    assert host_model.lib.hm_packed_slot_bytes(64 * 8) == 8192             # from 8 KiB on: whole KiB
+    assert host_model.lib.hm_packed_slot_bytes(71 * 8) == 9216
+    assert host_model.lib.hm_packed_slot_bytes(138 * 8) == 18432
+    assert host_model.lib.hm_packed_slot_bytes(1024 * 8) == FIFO_ENTRY_BYTES  # the longest run there is
+    for cu in (16, 256):
+        for cp in (1, 2, 3, 8, 16, 32):
+            max_ch = host_model.max_channel_count(cp, cu)
+            quarter = FIFO_ENTRY_BYTES * cp * max_ch
+            for run_channels in sorted({1, 2, max_ch}):
+                for lines in (1, 36, 63, 64, 71, 138, 1000, 1024):
+                    slot = host_model.lib.hm_packed_slot_bytes(lines * 8)
+                    assert slot >= lines * 128
+                    offs = sorted(host_model.stream_fifo_offset(s, ch, run_channels, lines, cp, cu)
+                                  for s in range(cp) for ch in range(run_channels))
+                    assert offs[0] == 0 and all(b - a >= slot for a, b in zip(offs, offs[1:]))
+                    assert offs[-1] + slot <= quarter
+                    for step in range(9):
+                        assert (host_model.stream_fifo_offset(cp - 1, run_channels - 1, run_channels, lines, cp, cu, step)
+                                == offs[-1] + (step % 4) * quarter)
+            assert 4 * quarter == FIFO_BYTES * cp * max_ch      # the four quarters are the reference's FIFO region
 
 
 def test_unit_to_piece_map_covers_every_piece_once(host_model):
@@ -133,23 +164,25 @@ def test_messages_of_a_run_are_packed_piece_by_piece(host_model):
     _, _, rc, msg = host_model.alltoall(ins_o, ins_s, ws, CU, 1, send=True, recv=False)
     assert rc == 0, msg
     max_ch = host_model.max_channel_count(cp, CU)
-    for sender in range(cp):
-        for receiver in range(cp):
-            off = host_model.lib.hm_fifo_offset(sender, 0, max_ch)
-            fifo = ws[receiver].view(np.uint64)[off // 8: (off + FIFO_BYTES) // 8]
-            lines = fifo[: 11 * 16].reshape(11, 16)
+    for receiver in range(cp):
+        region = ws[receiver].view(np.uint64)[: FIFO_BYTES * cp * max_ch // 8]
+        untouched = np.ones(region.size, dtype=bool)
+        for sender in range(cp):
+            off = host_model.stream_fifo_offset(sender, 0, 1, 11, cp, CU)
+            lines = region[off // 8: off // 8 + 11 * 16].reshape(11, 16)
+            untouched[off // 8: off // 8 + 11 * 16] = False
             run = np.concatenate([np.concatenate([ins_o[sender][e, receiver].view(np.uint64),
                                                   ins_s[sender][e, receiver].view(np.uint64)]) for e in range(entries)])
             assert run.size == 165
             assert (lines[:, :15].reshape(-1) == run).all()          # message after message, no gaps
             assert (lines[:, 15] == 0).all()                         # every line carries the step
-            assert (fifo[11 * 16:] == np.uint64(0xFFFFFFFFFFFFFFFF)).all()
+        assert (region[untouched] == np.uint64(0xFFFFFFFFFFFFFFFF)).all()
     # six messages: 198 pieces = 13.2 lines -> 14 lines, the last one zero padded
     ins_o, ins_s = random_inputs(cp, 6, x, s, seed=3)
     ws = host_model.new_workspace(cp, CU)
     out_o, out_s, rc, msg = host_model.alltoall(ins_o, ins_s, ws, CU, 1)
     assert rc == 0, msg
-    fifo = ws[1].view(np.uint64)[: FIFO_BYTES // 8]                  # sender 0 -> receiver 1
+    fifo = ws[1].view(np.uint64)[: 16384 // 8]                       # sender 0 -> receiver 1: the first 16 KiB slot
     last = fifo[13 * 16: 14 * 16]
     assert (last[3:15] == 0).all() and last[15] == 0 and (fifo[14 * 16:] == np.uint64(0xFFFFFFFFFFFFFFFF)).all()
     want_o, want_s = ho.exchange_closed_form(ins_o), ho.exchange_closed_form(ins_s)
@@ -184,10 +217,12 @@ def test_repeated_calls_reuse_entries_with_new_steps(host_model):
     so = host_model.lib.hm_sender_info_offset(cp, max_ch, 1, 1)
     assert ws[0][so // 8] == 9 and ws[0][so // 8 + 1] == 9  # one entry per call and stream
     # the flag of the first line of FIFO entry 9 % 4 == 1 ... entry 0 was last written at step 8
-    off = host_model.lib.hm_fifo_offset(0, 1, max_ch)
-    fifo = ws[1].view(np.uint64)[off // 8: (off + FIFO_BYTES) // 8]
-    assert fifo[15] == 8
-    assert fifo[FIFO_ENTRY_BYTES // 8 + 15] == 5
+    # (5 entries over 2 channels: channel 0 carries 3 messages of 17 pieces = 4 lines, the largest run of the launch)
+    row1 = ws[1].view(np.uint64)
+    assert row1[host_model.stream_fifo_offset(0, 1, 2, 4, cp, CU, step=8) // 8 + 15] == 8
+    assert row1[host_model.stream_fifo_offset(0, 1, 2, 4, cp, CU, step=5) // 8 + 15] == 5
+    assert (host_model.stream_fifo_offset(0, 1, 2, 4, cp, CU, step=5) - host_model.stream_fifo_offset(0, 1, 2, 4, cp, CU, step=8)
+            == FIFO_ENTRY_BYTES * cp * max_ch)   # a quarter of the FIFO region between consecutive positions
 
 
 def test_rounds_when_traffic_exceeds_the_fifo(host_model):
