@@ -217,7 +217,7 @@ __device__ __forceinline__ void fetch_scalars_up_front(const KernelArgs& a) {
   asm volatile("" ::"s"(a.parts), "s"(a.team), "s"(a.np0), "s"(a.np), "s"(a.msgsPerEntry), "s"(a.baseMsgs),
                "s"(a.extraChannels), "s"(a.byParts.magic), "s"(a.byParts.shift), "s"(a.byTeam.magic), "s"(a.byTeam.shift),
                "s"(a.byCp.magic), "s"(a.byCp.shift), "s"(a.byChannels.magic), "s"(a.byChannels.shift), "s"(a.sendBlocks), "s"(a.wavesPerBlock), "s"(a.dirBlocks), "s"(a.xcdGroup),
-               "s"(a.spinLimitTicks), "s"(a.slotBytes), "s"(a.positionBytes));
+               "s"(a.spinLimitTicks), "s"(a.slotBytes), "s"(a.positionBytes), "s"(a.positionMask));
 }
 
 // What a stream's wavefront needs to know, all wave-uniform.
@@ -395,7 +395,7 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
       }
       if (!opened && !open_entry()) return;
       if (U0 == slice.begin && firstMsg == 0) HELIX_MARK(wave, 1, true);
-      const uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * a.positionBytes;
+      const uint32_t entryOffset = (static_cast<uint32_t>(step) & a.positionMask) * a.positionBytes;
       const uint32_t stepLo = static_cast<uint32_t>(step);
       const uint32_t stepHi = static_cast<uint32_t>(static_cast<uint64_t>(step) >> 32);
 #pragma unroll
@@ -500,7 +500,7 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
       if (step < 0) return;
     }
     asm volatile("" ::: "memory");  // no line is read before the token was seen
-    const uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * a.positionBytes;
+    const uint32_t entryOffset = (static_cast<uint32_t>(step) & a.positionMask) * a.positionBytes;
     const uint32_t stepLo = static_cast<uint32_t>(step);
     const uint32_t stepHi = static_cast<uint32_t>(static_cast<uint64_t>(step) >> 32);
     for (uint32_t U0 = slice.begin; U0 < slice.end; U0 += kUnitsInFlight * kWaveLanes) {
@@ -693,7 +693,8 @@ struct CombineCtx {
   uint32_t channelBase;          // byte offset of sender 0's FIFO of this channel
   uint32_t senderStride;         // bytes between the FIFOs of consecutive senders
   uint32_t stepLo;               // lane q: step counter (low word) of sender q's stream
-  uint32_t positionBytes;        // bytes between the four positions an entry of a stream rotates through
+  uint32_t positionBytes;        // bytes between the positions an entry of a stream rotates through
+  uint32_t positionMask;         // positions of this launch - 1
 };
 
 template <int kLanesPerSlot>
@@ -706,7 +707,7 @@ __device__ __forceinline__ float shuffle_xor(float v, int mask) { return __shfl_
 
 // byte offset of sender q's open FIFO entry inside the receiver's FIFO region
 __device__ __forceinline__ uint32_t entry_base(const CombineCtx& cx, int q, uint32_t stepLo) {
-  return cx.channelBase + static_cast<uint32_t>(q) * cx.senderStride + (stepLo & (kFifoDepth - 1)) * cx.positionBytes;
+  return cx.channelBase + static_cast<uint32_t>(q) * cx.senderStride + (stepLo & cx.positionMask) * cx.positionBytes;
 }
 
 // byte offset of run piece g inside a FIFO entry: line g / 15, word g % 15
@@ -772,6 +773,7 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
   cx.channelBase = static_cast<uint32_t>(stream_fifo_offset(0, ch, a.runChannels, a.slotBytes));
   cx.senderStride = static_cast<uint32_t>(stream_fifo_offset(1, 0, a.runChannels, a.slotBytes));
   cx.positionBytes = a.positionBytes;
+  cx.positionMask = a.positionMask;
   __amdgpu_buffer_rsrc_t outRsrc = make_rsrc(a.rank[r].recv0, a.recvBytes0);
   __amdgpu_buffer_rsrc_t lseRsrc = make_rsrc(a.rank[r].recv1, a.rank[r].recv1 ? a.recvBytes1 : 0u);
   const unsigned long long lanesUpToMe = (2ull << lane) - 1ull;  // lanes 0..lane
@@ -1042,6 +1044,8 @@ static void set_launch_constants(KernelArgs& a) {
   a.extraChannels = entries % a.runChannels;
   a.entriesBase = entries_for_msgs(a.baseMsgs, sh);
   a.entriesExtra = entries_for_msgs(a.baseMsgs + 1, sh);
+  const int entriesPerStream = a.extraChannels > 0 ? a.entriesExtra : a.entriesBase;
+  a.positionMask = static_cast<uint32_t>(fifo_positions(exchange_lines_bytes(a.cpSize, a.runChannels, largest_run_units(a)), entriesPerStream)) - 1u;
   a.slotBytes = packed_slot_bytes(largest_run_units(a));
   a.positionBytes = fifo_position_bytes(a.cpSize, a.maxChannels);
   a.byParts = fast_div(static_cast<uint32_t>(a.parts));

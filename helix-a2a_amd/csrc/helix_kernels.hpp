@@ -50,6 +50,7 @@ struct KernelArgs {
   int dirBlocks;            // workgroups per direction (combine kernel: that send)
   int xcdGroup;             // consecutive workgroups' worth of streams that one XCD serves (xcd_grouped), 0: as dispatched
   uint32_t slotBytes;       // packed_slot_bytes(largest run of the launch): the streams of the launch sit this far apart
+  uint32_t positionMask;    // fifo_positions(...) - 1: the entry of step k sits in quarter k & positionMask
   uint32_t positionBytes;   // fifo_position_bytes: between the four positions (quarters of the FIFO region) an entry rotates through
   uint64_t spinLimitTicks;  // bound of one in-kernel wait, in 100 MHz ticks
   uint32_t* status;         // device status word (HELIX_A2A_STATUS_* bits)

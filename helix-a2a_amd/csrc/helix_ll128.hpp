@@ -34,7 +34,8 @@
 //   r, the receiver's counters in row r indexed by s, as in the reference.
 //   Where the stream's lines live inside row r's FIFO region is this build's
 //   own (nothing outside the kernels reads them): the region is four quarters,
-//   one per position a stream's entry rotates through (step & 3), and inside a
+//   one per position a stream's entry rotates through (step & 3; launches too
+//   large for the memory-side cache use fewer, see fifo_positions), and inside a
 //   quarter a launch packs its streams side by side, a slot of
 //   packed_slot_bytes(largest run of the launch) each -- see stream_fifo_offset.
 //   (The reference gives every stream four 128 KiB entries of its own,
@@ -96,7 +97,7 @@ HELIX_HD uint64_t workspace_bytes(int cpSize, int maxCh) {
 }
 
 // ---- where a launch puts its runs inside the receiver row's FIFO region ----------
-// A stream's entry of step k sits in quarter k & 3 of the region; a quarter is cp * maxCh * 128 KiB, room for a
+// A stream's entry of step k sits in quarter k & (positions - 1) of the region (fifo_positions below); a quarter is cp * maxCh * 128 KiB, room for a
 // full 128 KiB entry of every stream the layout provides for. Within the quarter the streams of a launch are
 // packed: stream (sender, channel) of a launch over runChannels channels starts at
 // (sender * runChannels + channel) * slotBytes, and slotBytes is the launch's largest run (every launch knows it:
@@ -111,6 +112,28 @@ HELIX_HD uint32_t packed_slot_bytes(long largestRunUnits) {
   const long bytes = largestRunUnits * kUnitBytes;
   if (bytes < 8192) return 16384;
   return static_cast<uint32_t>((bytes + 1023) / 1024 * 1024);  // at most kFifoEntryBytes: a run is at most 1024 lines
+}
+// How many of the four quarters the entries of a launch rotate through (1, 2 or 4; the entry of step k sits in
+// quarter k & (positions - 1)). Lines are dead once they have been received, but a cache does not know that:
+// every position a launch writes for the first time in a while pushes as many dead bytes of an older position
+// out of the 256 MB memory-side cache to DRAM. A launch whose lines of all four positions, with the tensors it
+// reads and writes (about as many bytes each as the lines), fit that cache keeps all four (24.2 us at cp = 8,
+// T = 256, against 27.5 us rewriting one position: lines that small are still in the L2s of the XCDs that read
+// them last); a larger one rewrites the same two, or the same one, every time (cp = 8, T = 512: 54.7 -> 44.9 us;
+// T = 768: 86.9 -> 65.8 us; c4: 99.4 -> 90.0 us). `linesBytes`: what the whole exchange writes into the FIFOs
+// of all ranks under one step, so that launches that carry a part of an exchange (one rank's send half) agree
+// with the others. A launch in which a stream opens more than one entry rotates through all four.
+constexpr uint64_t kMemorySideCacheBytes = 256ull << 20;
+HELIX_HD int fifo_positions(uint64_t linesBytes, int entriesPerStream) {
+  if (entriesPerStream > 1) return kFifoDepth;
+  const uint64_t budget = kMemorySideCacheBytes / 16 * 15;
+  if (6 * linesBytes <= budget) return 4;  // four positions of lines + tensors in + tensors out
+  if (4 * linesBytes <= budget) return 2;
+  return 1;
+}
+// bytes the streams of all cp * cp * runChannels (sender, receiver, channel) triples write under one step, at most
+HELIX_HD uint64_t exchange_lines_bytes(int cpSize, int runChannels, long largestRunUnits) {
+  return static_cast<uint64_t>(cpSize) * cpSize * runChannels * static_cast<uint64_t>(largestRunUnits) * kUnitBytes;
 }
 // byte offset of the stream's slot inside a quarter of the RECEIVER's row
 HELIX_HD uint64_t stream_fifo_offset(int sender, int channel, int runChannels, uint32_t slotBytes) {

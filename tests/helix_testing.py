@@ -66,7 +66,9 @@ class HostModel:
         lib.hm_alltoall.restype = ctypes.c_int
         lib.hm_last_message.restype = ctypes.c_char_p
         lib.hm_stream_fifo_offset.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_long, ctypes.c_int,
-                                              ctypes.c_int, ctypes.c_long]
+                                              ctypes.c_int, ctypes.c_long, ctypes.c_int]
+        lib.hm_fifo_positions.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_long, ctypes.c_int]
+        lib.hm_fifo_positions.restype = ctypes.c_int
         lib.hm_stream_fifo_offset.restype = ctypes.c_uint64
         lib.hm_packed_slot_bytes.argtypes = [ctypes.c_long]
         lib.hm_packed_slot_bytes.restype = ctypes.c_uint32
@@ -100,11 +102,13 @@ class HostModel:
         self.lib = lib
 
     def stream_fifo_offset(self, sender: int, channel: int, run_channels: int, largest_run_lines: int, cp: int,
-                           cu_count: int, step: int = 0) -> int:
+                           cu_count: int, step: int = 0, entries_per_stream: int = 1) -> int:
         """Byte offset inside the receiver's row of the lines stream (sender, channel) writes under ``step`` in a launch
-        over ``run_channels`` channels whose largest run has ``largest_run_lines`` lines."""
+        over ``run_channels`` channels whose largest run has ``largest_run_lines`` lines and whose streams open
+        ``entries_per_stream`` entries at most."""
+        positions = self.lib.hm_fifo_positions(cp, run_channels, largest_run_lines * 8, entries_per_stream)
         return self.lib.hm_stream_fifo_offset(sender, channel, run_channels, largest_run_lines * 8, cp,
-                                              self.max_channel_count(cp, cu_count), step)
+                                              self.max_channel_count(cp, cu_count), step, positions)
 
     def split_for_run(self, run_units: int, units_per_part: int = 6, max_parts: int = 16) -> Tuple[int, int]:
         """(wavefronts per stream, units in flight) the launch rule picks for a largest run of ``run_units`` units."""

@@ -51,6 +51,7 @@ struct Ctx {
   int unitsInFlight;   // per round, by the library's rule
   int parts;           // wavefronts that share a stream's runs, by the library's rule
   bool alignedStores;  // receivers of long runs store realigned 16-byte pieces
+  uint32_t positionMask;              // positions the round's entries rotate through - 1 (fifo_positions)
   uint32_t slotBytes, positionBytes;  // where the round's streams put their lines (packed_slot_bytes, fifo_position_bytes)
   // the FIFO region of rank r's row
   Extent fifoRegion(int r) const {
@@ -125,7 +126,7 @@ void run_sender(Ctx& c, int s, int r, int ch, int part) {
                (long long)step);
       return;
     }
-    uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * c.positionBytes;
+    uint32_t entryOffset = (static_cast<uint32_t>(step) & c.positionMask) * c.positionBytes;
     // tighter than the GPU's descriptor: every access must stay inside the stream's slot of this step's quarter
     Extent fifoExt{fifo + entryOffset, c.slotBytes};
     if (!c.chk.ok(c.fifoRegion(r), fifoExt.base, c.slotBytes, "fifo slot")) return;
@@ -183,7 +184,7 @@ void run_receiver(Ctx& c, int r, int s, int ch, int part) {
                  part, (long long)*token, (long long)step);
       return;
     }
-    uint32_t entryOffset = static_cast<uint32_t>(step & (kFifoDepth - 1)) * c.positionBytes;
+    uint32_t entryOffset = (static_cast<uint32_t>(step) & c.positionMask) * c.positionBytes;
     Extent fifoExt{fifo + entryOffset, c.slotBytes};
     if (!c.chk.ok(c.fifoRegion(r), fifoExt.base, c.slotBytes, "fifo slot")) return;
     uint8_t* base0 = const_cast<uint8_t*>(e0.base);
@@ -315,6 +316,8 @@ int hm_alltoall(const helix_a2a_params_t* per_rank, int cp, int cu_count, int ch
       c.parts = split.parts;
       c.unitsInFlight = split.unitsInFlight;
       c.alignedStores = maxRun > static_cast<long>(kMaxUnitsInFlight) * kWaveLanes;
+      const int msgsMax = stream_msg_count(c.entryBegin, c.entryEnd, 0, channels);
+      c.positionMask = static_cast<uint32_t>(fifo_positions(exchange_lines_bytes(cp, channels, maxRun), entries_for_msgs(msgsMax, c.sh))) - 1u;
       c.slotBytes = packed_slot_bytes(maxRun);
       c.positionBytes = fifo_position_bytes(cp, c.maxCh);
     }
@@ -346,9 +349,14 @@ int hm_split_for_run(long runUnits, int unitsPerPart, int maxParts) {
 // geometry probes for tests
 // byte offset, inside the receiver's row, of the lines stream (sender, channel) writes under step `step` in a launch
 // over `run_channels` channels whose largest run has `largest_run_units` units
-uint64_t hm_stream_fifo_offset(int sender, int channel, int run_channels, long largest_run_units, int cp, int max_ch, long step) {
+// (`positions`: fifo_positions of the launch)
+uint64_t hm_stream_fifo_offset(int sender, int channel, int run_channels, long largest_run_units, int cp, int max_ch, long step,
+                               int positions) {
   return stream_fifo_offset(sender, channel, run_channels, packed_slot_bytes(largest_run_units)) +
-         static_cast<uint64_t>(step & (kFifoDepth - 1)) * fifo_position_bytes(cp, max_ch);
+         static_cast<uint64_t>(step & (positions - 1)) * fifo_position_bytes(cp, max_ch);
+}
+int hm_fifo_positions(int cp, int run_channels, long largest_run_units, int entries_per_stream) {
+  return fifo_positions(exchange_lines_bytes(cp, run_channels, largest_run_units), entries_per_stream);
 }
 uint32_t hm_packed_slot_bytes(long largest_run_units) { return packed_slot_bytes(largest_run_units); }
 uint64_t hm_sender_info_offset(int cp, int max_ch, int receiver, int channel) {

@@ -636,6 +636,40 @@ def test_fifo_image_matches_host_model(hx, ops, host_model):
     check_against_oracle(dev_o, dev_s, out_o, out_s)
 
 
+def test_launches_of_different_sizes_alternate_on_one_workspace(hx, ops):
+    # the lines of a launch are packed by its own shape, and a launch too large for the memory-side cache rewrites
+    # one or two positions instead of rotating through four: launches of all three kinds follow each other on one
+    # workspace, fresh payload every time, exchange and fused combine
+    cp = 8
+    ws = get_workspace(hx, cp)
+    g = torch.Generator().manual_seed(91)
+    shapes = [(512, 1024, 16), (64, 1024, 16), (384, 1024, 16), (512, 1024, 16), (5, 256, 4), (384, 1024, 16), (512, 1024, 16)]
+    for rep, (entries, x, s) in enumerate(shapes):
+        ins_o = [torch.randint(-32768, 32767, (entries, cp, x), generator=g, dtype=torch.int16).view(torch.bfloat16).cuda()
+                 for _ in range(cp)]
+        ins_s = [torch.randint(-2**31, 2**31 - 1, (entries, cp, s), generator=g, dtype=torch.int32).view(torch.float32).cuda()
+                 for _ in range(cp)]
+        for _ in range(2):   # twice in a row: the second call rewrites (one position) or moves on (two, four)
+            outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws)
+        torch.cuda.synchronize()
+        assert_clean(ops)
+        check_against_oracle(ins_o, ins_s, outs_o, outs_s, with_numpy=False)
+        if rep % 2 == 0:
+            vals = [torch.randn(entries, cp, x, generator=g).to(torch.bfloat16).cuda() for _ in range(cp)]
+            lse = [torch.randn(entries, cp, s, generator=g).cuda() for _ in range(cp)]
+            combined = hx.alltoall_combine_loopback(vals, lse, ws, hx.STATS_LSE)
+            torch.cuda.synchronize()
+            assert_clean(ops)
+            heads = s // 2
+            recv_o = ho.exchange_closed_form([torch_bits(t) for t in vals])
+            recv_s = ho.exchange_closed_form([torch_bits(t) for t in lse])
+            for r in (0, cp - 1):
+                with np.errstate(all="ignore"):
+                    want, _ = ho.combine_after_exchange(ho.bf16_bits_to_f32(recv_o[r]), recv_s[r].view(np.float32), heads, 0)
+                got = combined[r].float().cpu().numpy()
+                assert (np.abs(got - want) <= 2e-2 + 2e-2 * np.abs(want)).all()
+
+
 # ---------------------------------------------------------------------------
 # bounded waits and back-pressure
 # ---------------------------------------------------------------------------

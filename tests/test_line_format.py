@@ -123,10 +123,26 @@ def test_packed_layout_keeps_the_streams_of_a_launch_apart(host_model):
                                   for s in range(cp) for ch in range(run_channels))
                     assert offs[0] == 0 and all(b - a >= slot for a, b in zip(offs, offs[1:]))
                     assert offs[-1] + slot <= quarter
+                    positions = host_model.lib.hm_fifo_positions(cp, run_channels, lines * 8, 1)
+                    assert positions in (1, 2, 4)
                     for step in range(9):
                         assert (host_model.stream_fifo_offset(cp - 1, run_channels - 1, run_channels, lines, cp, cu, step)
-                                == offs[-1] + (step % 4) * quarter)
+                                == offs[-1] + (step % positions) * quarter)
+                        assert (host_model.stream_fifo_offset(cp - 1, run_channels - 1, run_channels, lines, cp, cu, step, 3)
+                                == offs[-1] + (step % 4) * quarter)     # several entries per stream: all four
             assert 4 * quarter == FIFO_BYTES * cp * max_ch      # the four quarters are the reference's FIFO region
+    # positions: all four while the lines of four positions and the tensors fit the memory-side cache, then two, then one;
+    # a launch in which a stream opens several entries always rotates through four
+    pos = host_model.lib.hm_fifo_positions
+    assert pos(8, 128, 36 * 8, 1) == 4          # c3: 37.7 MB of lines per launch
+    assert pos(8, 128, 54 * 8, 1) == 2          # cp = 8, T = 384: 56.6 MB
+    assert pos(8, 128, 71 * 8, 1) == 1          # cp = 8, T = 512: 74.4 MB
+    assert pos(8, 128, 138 * 8, 1) == 1         # c4: 144.7 MB
+    assert pos(16, 64, 71 * 8, 1) == 1          # c5a: 148.9 MB
+    assert pos(8, 128, 138 * 8, 2) == 4 and pos(2, 1, 1024 * 8, 4) == 4
+    assert pos(2, 8, 9 * 8, 1) == 4             # c1
+    big = host_model.stream_fifo_offset(1, 2, 128, 138, 8, 256, step=7)
+    assert big == host_model.stream_fifo_offset(1, 2, 128, 138, 8, 256, step=0)   # one position: every step in place
 
 
 def test_unit_to_piece_map_covers_every_piece_once(host_model):
