@@ -69,9 +69,10 @@ constexpr int kAuxSc1 = 16;
 constexpr uint32_t kRsrcWord3 = 0x00020000u;   // raw buffer, 32-bit data format
 constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any descriptor (extents are < 2 GiB)
 
-// Both kernels are held to four wavefronts per SIMD (16 per CU): with more
-// resident wavefronts the same traffic takes 1-5 % longer on MI355X, on every
-// shape measured, whatever the register count would allow.
+// Launches of independent wavefronts and the combine kernel are held to four
+// wavefronts per SIMD (16 per CU): with more resident wavefronts the same
+// traffic takes 1-5 % longer on MI355X, on every shape measured, whatever the
+// register count would allow. (Teams of the exchange kernel run at six, see there.)
 #define HELIX_WAVES_PER_SIMD __attribute__((amdgpu_waves_per_eu(4, 4)))
 
 constexpr int kDppWaveShl1 = 0x130;  // DPP control: lane i reads lane i + 1 of the wavefront
@@ -618,8 +619,11 @@ __device__ __forceinline__ void run_sender_any(const KernelArgs& a, int s, int r
 // Within a direction, w = ((local rank * runChannels + channel) * cp + peer) * parts + part:
 // neighbouring wavefronts touch neighbouring slices, then neighbouring rows of the same entry.
 // With kTeam a workgroup is one team: workgroup b serves stream b of the launch (parts = 1).
+// (Teams run six wavefronts per SIMD instead of four: a workgroup is then a team of 3..8 wavefronts, and sixteen
+// slots per CU hold only five teams of three, or three of five; with 24 slots c4's teams of three measured 88.5 ->
+// 85.4 us, teams of five 140 -> 101 us. Launches of independent wavefronts stay at four, where 5, 6 and 8 are slower.)
 template <int kUnitsInFlight, bool kAlignedStores, bool kTeam>
-__global__ __launch_bounds__(1024) HELIX_WAVES_PER_SIMD void helix_exchange_kernel(KernelArgs a) {
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(kTeam ? 6 : 4, kTeam ? 6 : 4))) void helix_exchange_kernel(KernelArgs a) {
   __shared__ TeamLds teamLds;
   fetch_scalars_up_front(a);
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWaveLanes);
