@@ -485,6 +485,9 @@ def main() -> int:
     ap.add_argument("--no-host-timing", action="store_true", help="skip the host-time-per-call measurements")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--no-distribution", action="store_true",
+                    help="skip the per-call event pairs behind the timed region (single_call_us): a kernel trace of the run "
+                         "then holds the warm-up and the timed launches only")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="also run 5 elementwise copies (read MIB, write MIB) so that a counter run can be scaled")
     args = ap.parse_args()
@@ -585,7 +588,7 @@ def main() -> int:
         avg_kernel_ms = _event_us(plan.run, roofline_steps, 0) * 1e-3
 
     # distribution of single calls (event pair per call), outside the timed region
-    n_dist = min(args.steps, 500)
+    n_dist = 0 if args.no_distribution else min(args.steps, 500)
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(n_dist)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(n_dist)]
     for i in range(n_dist):
@@ -683,7 +686,7 @@ def main() -> int:
         # payload read + result written over the time per call: what a direct permuted copy would have to move;
         # `value` counts the FIFO write and read-back as well (the protocol's own traffic)
         "payload_GBps": useful_bytes / (ms_per_step * 1e-3) / 1e9,
-        "single_call_us": {
+        "single_call_us": None if not kernel_ms else {
             "mean": statistics.fmean(kernel_ms) * 1e3,
             "p50": percentile(kernel_ms, 0.5) * 1e3,
             "p5": percentile(kernel_ms, 0.05) * 1e3,

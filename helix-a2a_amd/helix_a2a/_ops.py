@@ -58,6 +58,18 @@ class _CombineOut(ctypes.Structure):
     _fields_ = [("combined", ctypes.c_void_p), ("lse_out", ctypes.c_void_p)]
 
 
+# A descriptor array seen as 8-byte words: a call that only swaps data pointers writes them as plain integers
+# (a C-level item assignment) instead of through four levels of ctypes attribute access.
+_PARAMS_WORDS = ctypes.sizeof(_Params) // 8
+_SEND0, _SEND1 = _Params.send_fields.offset // 8, (_Params.send_fields.offset + ctypes.sizeof(_Field)) // 8
+_RECV0, _RECV1 = _Params.recv_fields.offset // 8, (_Params.recv_fields.offset + ctypes.sizeof(_Field)) // 8
+assert ctypes.sizeof(_Params) % 8 == 0 and _Field.data.offset == 0 and ctypes.sizeof(_CombineOut) == 16
+
+
+def _words(arr: ctypes.Array) -> ctypes.Array:
+    return (ctypes.c_uint64 * (ctypes.sizeof(arr) // 8)).from_buffer(arr)
+
+
 def _load_library() -> ctypes.CDLL:
     path = Path(os.environ.get("HELIX_A2A_LIBRARY", Path(__file__).resolve().parent / _LIB_NAME))
     if not path.exists():
@@ -304,10 +316,11 @@ class _ExchangeShape:
         self.shape_o = partial_o.shape
         self.shape_s = softmax_stats.shape
         self.dtype = partial_o.dtype
-        self.arrays: Dict[tuple, ctypes.Array] = {}
+        self.arrays: Dict[tuple, Tuple[ctypes.Array, ctypes.Array]] = {}
 
-    def array(self, workspace: torch.Tensor, channel_count: int) -> ctypes.Array:
-        """The cp descriptors of this shape on this workspace, everything but the data pointers filled in."""
+    def array(self, workspace: torch.Tensor, channel_count: int) -> Tuple[ctypes.Array, ctypes.Array]:
+        """The cp descriptors of this shape on this workspace, everything but the data pointers filled in, and
+        the same memory as 8-byte words."""
         key = (workspace.data_ptr(), workspace.stride(0), channel_count)
         arr = self.arrays.get(key)
         if arr is None:
@@ -326,7 +339,7 @@ class _ExchangeShape:
                 p.workspace_stride_u64 = key[1]
                 p.cp_rank, p.cp_size = r, self.cp_size
                 p.channel_count, p.max_channel_count = int(channel_count), max_ch
-            self.arrays[key] = arr
+            arr = self.arrays[key] = (arr, _words(arr))
         return arr
 
 
@@ -414,7 +427,7 @@ class _LogicalRankGroup:
     call and used for every launch of it, whatever the environment says later.
     """
 
-    __slots__ = ("cp_size", "pending", "streams", "shape", "arr", "eager", "started", "workspace", "outs_o", "outs_s")
+    __slots__ = ("cp_size", "pending", "streams", "shape", "arr", "words", "eager", "started", "workspace", "outs_o", "outs_s")
 
     def __init__(self, cp_size: int) -> None:
         self.cp_size = cp_size
@@ -427,6 +440,7 @@ class _LogicalRankGroup:
         self.streams.clear()
         self.shape: Optional[_ExchangeShape] = None
         self.arr: Optional[ctypes.Array] = None
+        self.words: Optional[ctypes.Array] = None
         self.eager = False
         self.started = 0.0
         self.workspace: Optional[torch.Tensor] = None
@@ -437,7 +451,7 @@ class _LogicalRankGroup:
         max_ch = _device_max_channels(self.cp_size)
         _require(channels <= max_ch, f"alltoall: channel_count {channels} exceeds max_channel_count {max_ch}")
         self.shape = shape
-        self.arr = shape.array(workspace, channels)
+        self.arr, self.words = shape.array(workspace, channels)
         self.eager = _eager_send
         self.started = time.monotonic()
         self.workspace = workspace  # kept while ranks are pending: the caller may have passed a temporary view
@@ -460,14 +474,14 @@ class _LogicalRankGroup:
         else:
             self._begin(shape, workspace)
         out_o, out_s = self.outs_o[rank], self.outs_s[rank]
-        p = self.arr[rank]
-        p.send_fields[0].data = partial_o.data_ptr()
-        p.send_fields[1].data = softmax_stats.data_ptr()
-        p.recv_fields[0].data = out_o.data_ptr()
-        p.recv_fields[1].data = out_s.data_ptr()
+        words, base = self.words, rank * _PARAMS_WORDS
+        words[base + _SEND0] = partial_o.data_ptr()
+        words[base + _SEND1] = softmax_stats.data_ptr()
+        words[base + _RECV0] = out_o.data_ptr()
+        words[base + _RECV1] = out_s.data_ptr()
         stream = _stream_handle()
         if self.eager:
-            rc = _lib.helix_a2a_alltoall_send(ctypes.byref(p), 1, stream)
+            rc = _lib.helix_a2a_alltoall_send(ctypes.byref(self.arr[rank]), 1, stream)
             if rc == 3 and not pending:  # HELIX_A2A_ERR_CAPACITY on the first rank: the fused launch and its rounds instead
                 self.eager = False
             elif rc != 0:
@@ -567,7 +581,7 @@ def alltoall_loopback(partial_o: Sequence[torch.Tensor], softmax_stats: Sequence
         outs_o, outs_s = list(out[0]), list(out[1])
         _require(len(outs_o) == cp_size and len(outs_s) == cp_size, "need one output pair per rank")
     with _call_lock, _on_device(device):
-        arr = shape.array(workspace, int(channel_count))
+        arr, words = shape.array(workspace, int(channel_count))
         for r in range(cp_size):
             o, st = partial_o[r], softmax_stats[r]
             if r > 0:
@@ -578,11 +592,11 @@ def alltoall_loopback(partial_o: Sequence[torch.Tensor], softmax_stats: Sequence
                 _require(oo.shape == o.shape and oo.dtype == o.dtype and oo.is_contiguous()
                          and os_.shape == st.shape and os_.dtype == torch.float32 and os_.is_contiguous()
                          and oo.is_cuda and os_.is_cuda, "out tensors must match the inputs")
-            p = arr[r]
-            p.send_fields[0].data = o.data_ptr()
-            p.send_fields[1].data = st.data_ptr()
-            p.recv_fields[0].data = oo.data_ptr()
-            p.recv_fields[1].data = os_.data_ptr()
+            base = r * _PARAMS_WORDS
+            words[base + _SEND0] = o.data_ptr()
+            words[base + _SEND1] = st.data_ptr()
+            words[base + _RECV0] = oo.data_ptr()
+            words[base + _RECV1] = os_.data_ptr()
         rc = _lib.helix_a2a_alltoall_loopback(arr, cp_size, _stream_handle())
     if rc != 0:
         _raise_last("alltoall_loopback")
@@ -745,6 +759,7 @@ class _ReduceDescriptors:
             p.cp_rank, p.cp_size = r, cp_size
             p.channel_count, p.max_channel_count = int(channel_count), max_ch
             self.out[r].lse_out = None
+        self.arr_words, self.out_words = _words(self.arr), _words(self.out)
 
 
 _reduce_descriptors: Dict[tuple, _ReduceDescriptors] = {}
@@ -772,9 +787,12 @@ def dcp_reduce(cp_attn_out: Sequence[torch.Tensor], cp_attn_lse: Sequence[torch.
     _require(h % n == 0, "H must be divisible by the rank count")
     hp = h // n
     _require(d % 4 == 0 and d >= 32, "head_dim must be a multiple of 4 and >= 32")
-    _check_workspace(workspace, n)
-    _require(workspace.device == device, "all tensors must live on one device")
-    key = (n, b, h, d, dtype, workspace.data_ptr(), workspace.stride(0), int(channel_count), device.index)
+    if not (isinstance(workspace, torch.Tensor) and workspace.dtype is torch.int64 and workspace.dim() == 2
+            and workspace.size(0) == n and workspace.stride(1) == 1 and workspace.is_cuda):
+        _check_workspace(workspace, n)  # says which of them it was
+    index = o0.get_device()
+    _require(workspace.get_device() == index, "all tensors must live on one device")
+    key = (n, b, h, d, dtype, workspace.data_ptr(), workspace.stride(0), int(channel_count), index)
     # one allocation per kind of output; rank r's result is slice r of it
     combined = torch.empty((n, b, hp, d), dtype=dtype, device=device).unbind(0)
     lses = torch.empty((n, b, hp), dtype=torch.float32, device=device).unbind(0) if return_lse else None
@@ -786,11 +804,14 @@ def dcp_reduce(cp_attn_out: Sequence[torch.Tensor], cp_attn_lse: Sequence[torch.
                 _reduce_descriptors.clear()
             desc = _reduce_descriptors[key] = _ReduceDescriptors(n, b, h, d, dtype, workspace, channel_count)
         arr, out = desc.arr, desc.out
+        arr_words, out_words = desc.arr_words, desc.out_words
+        combined_ptr, combined_step = combined[0].data_ptr(), b * hp * d * combined[0].element_size()
+        lse_ptr, lse_step = (lses[0].data_ptr(), b * hp * 4) if return_lse else (0, 0)
         for r in range(n):
             o, lse = cp_attn_out[r], cp_attn_lse[r]
-            if not (o.shape == shape and o.dtype == dtype and o.device == device):
+            if not (o.shape == shape and o.dtype is dtype and o.get_device() == index):
                 raise RuntimeError("all ranks must pass cp_attn_out of one shape, dtype and device")
-            if not (lse.shape == lse_shape and lse.dtype == torch.float32 and lse.device == device):
+            if not (lse.shape == lse_shape and lse.dtype is torch.float32 and lse.get_device() == index):
                 raise RuntimeError("cp_attn_lse must be float32 [B, H] on the same device")
             if not o.is_contiguous():
                 o = o.contiguous()
@@ -798,11 +819,10 @@ def dcp_reduce(cp_attn_out: Sequence[torch.Tensor], cp_attn_lse: Sequence[torch.
             if not lse.is_contiguous():
                 lse = lse.contiguous()
                 keep.append(lse)
-            fields = arr[r].send_fields
-            fields[0].data = o.data_ptr()
-            fields[1].data = lse.data_ptr()
-            out[r].combined = combined[r].data_ptr()
-            out[r].lse_out = lses[r].data_ptr() if return_lse else None
+            arr_words[r * _PARAMS_WORDS + _SEND0] = o.data_ptr()
+            arr_words[r * _PARAMS_WORDS + _SEND1] = lse.data_ptr()
+            out_words[2 * r] = combined_ptr + r * combined_step
+            out_words[2 * r + 1] = lse_ptr + r * lse_step
         mode = STATS_LSE_PACKED | (STATS_BASE2 if lse_base2 else 0)
         rc = _lib.helix_a2a_alltoall_combine_loopback(arr, out, n, mode, desc.dtype_code, _stream_handle())
     if rc != 0:
