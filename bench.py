@@ -352,8 +352,8 @@ def chunk_copy_probe(names=("c3", "c4", "c5a"), reps: int = 40, kernel_us=None):
     """What a plain chunked copy of each workload's shape reaches on this box (helix-a2a_amd/benchmark/memory_probe.hip):
     one chunk per stream, as long as the stream's run of LL128 lines, moved by as many wavefronts as the exchange
     kernel gives a run, in the same passes of 16-byte units -- no counters, tokens, flags or index arithmetic.
-    `send`: dense memory -> FIFO-like slots 512 KiB apart (the entry of a slot rotating through its four positions,
-    as the FIFOs' do); `recv`: slots -> dense. Hot re-uses one dense buffer per side, cold takes the next of N
+    `send`: dense memory -> slots placed as the kernels place a launch's runs (side by side, rotating through the
+    same number of positions); `recv`: slots -> dense. Hot re-uses one dense buffer per side, cold takes the next of N
     (1 GiB in rotation). `copy_bound_us` = send + recv, each scaled from the probe's bytes (lines in, lines out) to
     the exchange's (payload + lines): the time the two halves of the exchange would take at the probe's rates.
     `kernel_us`: {workload: (hot, cold)} of the exchange kernel, to put beside it."""
@@ -370,7 +370,6 @@ def chunk_copy_probe(names=("c3", "c4", "c5a"), reps: int = 40, kernel_us=None):
     lib.helix_probe_chunk_copy.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_uint64,
                                            ctypes.c_uint32, ctypes.c_uint32, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
     lib.helix_probe_chunk_copy.restype = ctypes.c_int
-    slot, entry = 512 * 1024, 128 * 1024
     out = {}
     for name in names:
         w = WORKLOADS[name]
@@ -387,7 +386,13 @@ def chunk_copy_probe(names=("c3", "c4", "c5a"), reps: int = 40, kernel_us=None):
         team = min(passes, 8) if passes >= 3 and 2 * streams > 4096 else 1   # the exchange kernel's rule for teams
         dense_bytes = streams * chunk
         n_sets = max(2, -(-(1 << 30) // (2 * dense_bytes)))
-        slots = torch.empty(streams * slot, dtype=torch.uint8, device="cuda")
+        # the exchange kernels' placement of a launch's runs: side by side, a slot each (the run rounded up to whole
+        # KiB, 16 KiB for runs below 8 KiB), in one of up to four positions a quarter of the FIFO region apart
+        # -- four while six times the lines fit 240 MB, two while four times do, else one
+        slot = 16384 if chunk < 8192 else -(-chunk // 1024) * 1024
+        positions = 4 if 6 * dense_bytes <= 240 << 20 else 2 if 4 * dense_bytes <= 240 << 20 else 1
+        entry = streams * slot
+        slots = torch.empty(positions * entry, dtype=torch.uint8, device="cuda")
         slots.fill_(1)
         dense = [torch.full((dense_bytes,), 2, dtype=torch.uint8, device="cuda") for _ in range(2 * n_sets)]
         stream = _ops._stream_handle()
@@ -397,7 +402,7 @@ def chunk_copy_probe(names=("c3", "c4", "c5a"), reps: int = 40, kernel_us=None):
             i = turn[0]
             turn[0] += 1
             d = dense[(2 * (i % n_sets) if cold else 0) + (0 if send else 1)]
-            s_ptr = slots.data_ptr() + (i % 4) * entry
+            s_ptr = slots.data_ptr() + (i % positions) * entry
             if send:
                 rc = lib.helix_probe_chunk_copy(d.data_ptr(), chunk, s_ptr, slot, chunk, streams, team, 0, stream)
             else:
@@ -405,12 +410,12 @@ def chunk_copy_probe(names=("c3", "c4", "c5a"), reps: int = 40, kernel_us=None):
             if rc != 0:
                 raise RuntimeError(f"helix_probe_chunk_copy failed: {rc}")
 
-        row = {"chunk_bytes": chunk, "chunks": streams, "wavefronts_per_chunk": team}
+        row = {"chunk_bytes": chunk, "chunks": streams, "wavefronts_per_chunk": team, "slot_bytes": slot, "positions": positions}
         scale = (w.payload_bytes / runs_per_stream + wire / runs_per_stream) / (2.0 * dense_bytes)  # exchange half / probe leg, in bytes
         for cold in (False, True):
             tag = "cold" if cold else "hot"
-            send_us = _event_us(lambda: leg(True, cold), reps, 2 * n_sets if cold else 5)
-            recv_us = _event_us(lambda: leg(False, cold), reps, 2 * n_sets if cold else 5)
+            send_us = _event_us(lambda: leg(True, cold), reps, 2 * n_sets if cold else 20)
+            recv_us = _event_us(lambda: leg(False, cold), reps, 2 * n_sets if cold else 20)
             row[tag] = {"send_us": send_us, "recv_us": recv_us,
                         "send_GBps": 2 * dense_bytes / send_us / 1e3, "recv_GBps": 2 * dense_bytes / recv_us / 1e3,
                         "copy_bound_us": (send_us + recv_us) * scale * runs_per_stream}
@@ -423,7 +428,7 @@ def chunk_copy_probe(names=("c3", "c4", "c5a"), reps: int = 40, kernel_us=None):
         del slots, dense
         torch.cuda.empty_cache()
     out["note"] = ("plain chunked copies of each workload's shape (one chunk per stream, its run of lines; dense <-> slots "
-                   "512 KiB apart), GB/s of bytes read + written; copy_bound_us = the two halves of the exchange at these rates")
+                   "placed like the kernels' runs), GB/s of bytes read + written; copy_bound_us = the two halves of the exchange at these rates")
     return out
 
 

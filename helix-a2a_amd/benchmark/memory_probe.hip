@@ -7,7 +7,7 @@
 // dst + c * dst_stride, by `waves_per_chunk` wavefronts that each take a contiguous slice of whole 1 KiB
 // wave accesses and walk it in passes of up to six 16-byte units per lane, all loads of a pass before its
 // first store -- what the exchange kernel's wavefronts do, without counters, tokens, flags, line format or
-// index arithmetic. Same occupancy (four wavefronts per SIMD), same buffer-descriptor accesses.
+// index arithmetic. Same occupancy (four wavefronts per SIMD, six for teams), same buffer-descriptor accesses.
 //
 // What this copy reaches on a shape is what the memory system gives chunk-per-wavefront traffic of that shape;
 // bench.py --probe chunk-copy puts the exchange kernels beside it. Measuring equipment: the product library
@@ -61,7 +61,9 @@ __device__ __forceinline__ void move_slice(const ProbeArgs& a, __amdgpu_buffer_r
   if (a.mode == 1 && (acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345678u) a.sink[0] = 1;  // keeps the loads alive
 }
 
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void helix_probe_chunk_copy_kernel(ProbeArgs a) {
+// kTeam: several wavefronts per chunk, one workgroup per chunk, six wavefronts per SIMD (as the exchange kernel's teams)
+template <bool kTeam>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(kTeam ? 6 : 4, kTeam ? 6 : 4))) void helix_probe_chunk_copy_kernel(ProbeArgs a) {
   const int wave = static_cast<int>(threadIdx.x) / kLanes, lane = static_cast<int>(threadIdx.x) % kLanes;
   const int wavesPerBlock = static_cast<int>(blockDim.x) / kLanes;
   uint32_t chunk;
@@ -120,7 +122,11 @@ extern "C" int helix_probe_chunk_copy(const void* src, uint64_t src_stride, void
   a.sink = static_cast<uint32_t*>(sink);
   const int wavesPerBlock = waves_per_chunk > 1 ? waves_per_chunk : 2;
   const uint32_t blocks = waves_per_chunk > 1 ? chunks : (chunks + wavesPerBlock - 1) / wavesPerBlock;
-  hipLaunchKernelGGL(helix_probe_chunk_copy_kernel, dim3(blocks), dim3(wavesPerBlock * kLanes), 0,
-                     static_cast<hipStream_t>(stream), a);
+  if (waves_per_chunk > 1)
+    hipLaunchKernelGGL(helix_probe_chunk_copy_kernel<true>, dim3(blocks), dim3(wavesPerBlock * kLanes), 0,
+                       static_cast<hipStream_t>(stream), a);
+  else
+    hipLaunchKernelGGL(helix_probe_chunk_copy_kernel<false>, dim3(blocks), dim3(wavesPerBlock * kLanes), 0,
+                       static_cast<hipStream_t>(stream), a);
   return static_cast<int>(hipGetLastError());
 }
