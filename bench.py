@@ -40,12 +40,12 @@ MIN_ROOFLINE_STEPS = 200
 # <kernel>_<workload>.md hold the runs these come from. These counters sit between L2 and fabric:
 # they do not tell whether the memory-side cache or DRAM served a request.
 MEASURED_TRAFFIC_BYTES = {
-    ("helix_exchange_kernel", "c3", 128): 151_031_722,   # profiles/helix_exchange_kernel_c3.md
-    ("helix_exchange_kernel", "c4", 128): 566_613_588,   # profiles/helix_exchange_kernel_c4.md
-    ("helix_exchange_kernel", "c5a", 64): 587_707_467,   # profiles/helix_exchange_kernel_c5a.md
-    ("helix_combine_kernel", "c3", 128): 118_789_868,    # profiles/helix_combine_kernel_c3.md
-    ("helix_combine_kernel", "c4", 128): 451_874_147,    # profiles/helix_combine_kernel_c4.md
-    ("helix_combine_kernel", "c5a", 64): 465_818_182,    # profiles/helix_combine_kernel_c5a.md
+    ("helix_exchange_kernel", "c3", 128): 150_946_519,   # profiles/helix_exchange_kernel_c3.md
+    ("helix_exchange_kernel", "c4", 128): 566_978_407,   # profiles/helix_exchange_kernel_c4.md
+    ("helix_exchange_kernel", "c5a", 64): 588_543_088,   # profiles/helix_exchange_kernel_c5a.md
+    ("helix_combine_kernel", "c3", 128): 118_757_998,   # profiles/helix_combine_kernel_c3.md
+    ("helix_combine_kernel", "c4", 128): 451_090_862,   # profiles/helix_combine_kernel_c4.md
+    ("helix_combine_kernel", "c5a", 64): 465_016_573,   # profiles/helix_combine_kernel_c5a.md
 }
 
 
@@ -194,7 +194,7 @@ def _graph_of(fn, calls: int):
 GRAPH_CALLS = 10  # exchanges per captured graph in the per-rank and decode-size rows: amortises the cost of a graph launch
 
 
-def per_rank_gpu_timing(names=("c2", "c3"), steps: int = 200, spare=None):
+def per_rank_gpu_timing(names=("c2", "c3"), steps: int = 200, spare=None, policies=(False, True)):
     """GPU time of the reference's signature: cp calls of helix_a2a.alltoall (one per logical rank) per exchange,
     beside the one fused call of all ranks. HIP events around back-to-back exchanges; `eager` is bounded below
     by what the Python calls cost the host, `graph` replays a captured graph of GRAPH_CALLS exchanges.
@@ -225,6 +225,8 @@ def per_rank_gpu_timing(names=("c2", "c3"), steps: int = 200, spare=None):
         row["loopback"]["graph"] = _event_us(graph.replay, max(steps // GRAPH_CALLS, 10), 3) / GRAPH_CALLS
         del graph, keep
         for policy, eager_send in (("alltoall_x_cp", False), ("alltoall_x_cp_eager_send", True)):
+            if eager_send not in policies:
+                continue
             _ops.set_eager_send(eager_send)
             try:
                 row[policy] = {"eager": _event_us(per_rank, steps, 30)}
@@ -233,7 +235,8 @@ def per_rank_gpu_timing(names=("c2", "c3"), steps: int = 200, spare=None):
                 del graph, keep
             finally:
                 _ops.set_eager_send(False)
-        row["alltoall_x_cp_over_loopback"] = {k: row["alltoall_x_cp"][k] / row["loopback"][k] for k in ("eager", "graph")}
+        if "alltoall_x_cp" in row:
+            row["alltoall_x_cp_over_loopback"] = {k: row["alltoall_x_cp"][k] / row["loopback"][k] for k in ("eager", "graph")}
         out[name] = row
         torch.cuda.synchronize()
         del plan, ins_o, ins_s, ws
@@ -484,6 +487,10 @@ def main() -> int:
     ap.add_argument("--team-units", type=int, default=None, metavar="U",
                     help="teams of wavefronts per stream: 1..6 always (at most U KiB per wavefront), 0 never, "
                          "-1 the library's rule (runs of three or more passes in launches that queue)")
+    ap.add_argument("--per-rank", choices=("fused", "eager-send", "both"), default=None,
+                    help="print only the GPU time of the reference's signature on --workload: cp calls of helix_a2a.alltoall "
+                         "per exchange, eager and replayed from a HIP graph, beside the one fused call; fused = the default "
+                         "(the last rank's call issues one launch), eager-send = every rank's send half at its call")
     ap.add_argument("--probe", choices=("chunk-copy",), default=None,
                     help="chunk-copy: print only the memory probe -- plain chunked copies of the shapes of c3, c4 and c5a, "
                          "hot and cold, beside the exchange kernel on the same workloads -- as one JSON line")
@@ -512,6 +519,10 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
     torch.cuda.set_device(0)
+    if args.per_rank:
+        policies = {"fused": (False,), "eager-send": (True,), "both": (False, True)}[args.per_rank]
+        print(json.dumps({"per_rank_gpu_us": per_rank_gpu_timing((args.workload,), max(args.steps, MIN_ROOFLINE_STEPS), policies=policies)}))
+        return 0 if _ops.device_status() == 0 else 1
     if args.probe == "chunk-copy":
         timings = {n: exchange_kernel_timing(WORKLOADS[n], max(args.steps, MIN_ROOFLINE_STEPS)) for n in ("c3", "c4", "c5a")}
         probe = chunk_copy_probe(kernel_us={n: (t["kernel_us"], t["kernel_us_cold"]) for n, t in timings.items()})

@@ -2,7 +2,7 @@
 // of their protocol.
 //
 // A stream's wavefront of the Helix exchange moves one run: a few KiB that are contiguous on the FIFO side
-// (slots 512 KiB apart, one per stream) and contiguous or in rows on the tensor side. This kernel moves
+// (a slot per stream) and contiguous or in rows on the tensor side. This kernel moves
 // `chunks` such chunks: chunk c is `chunk_bytes` long, read at src + c * src_stride and written at
 // dst + c * dst_stride, by `waves_per_chunk` wavefronts that each take a contiguous slice of whole 1 KiB
 // wave accesses and walk it in passes of up to six 16-byte units per lane, all loads of a pass before its
