@@ -12,8 +12,12 @@ On one GPU the ``cp_size`` context-parallel ranks are logical ranks: row ``r``
 of the workspace tensor is rank ``r``'s FIFO memory, and all rows live in the
 same HBM. ``alltoall`` is called once per logical rank; the outputs of every
 rank are complete once all ``cp_size`` ranks have made their call and the
-stream has drained -- the single-device form of "every rank takes part".
-``alltoall_loopback`` issues all ranks in one fused launch.
+stream has drained -- the single-device form of "every rank takes part" -- and
+a rank's inputs belong to the exchange until then: the last rank's call issues
+the exchange of all ranks as one fused launch. (``HELIX_A2A_EAGER_SEND=1``:
+every rank's call launches its send half at once, and its inputs may be
+overwritten in stream order right after, at the price of ``cp_size + 1``
+launches per exchange.) ``alltoall_loopback`` issues all ranks in one call.
 """
 from __future__ import annotations
 
@@ -96,7 +100,9 @@ def alltoall(
     ``[..., cp_size, S]`` (fp32, S even); slice ``[..., p, :]`` goes to rank
     ``p``. Returns tensors of the same shapes whose slice ``[..., p, :]`` came
     from rank ``p``: ``out_r[e, s, :] = in_s[e, r, :]``, bit for bit.
-    Asynchronous on the current stream.
+    Asynchronous on the current stream. With the ranks of one device the
+    returned tensors are filled once every rank has called (see the module
+    docstring for what that asks of the inputs).
     """
     return _ops.alltoall_native(partial_o, softmax_stats, workspace, cp_rank, cp_size)
 
