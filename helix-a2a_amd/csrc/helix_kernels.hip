@@ -170,6 +170,16 @@ __device__ __forceinline__ uint64_t broken_at_launch(const KernelArgs& a) {
   return *reinterpret_cast<ConstWord*>(reinterpret_cast<uintptr_t>(broken_word(a)));
 }
 
+// A counter as it stood when this launch started (what the launches before it left), read through the scalar
+// cache like the broken word: wave-uniform, off the vector memory pipeline, so that it neither takes vector
+// registers nor sits in the queue of vector loads that the payload loads and their waits go through. Only for
+// counters that nothing in the running launch moves before this wavefront is done reading them (a stream's own
+// step, the tail a sender starts from); everything a wavefront polls goes through ld_counter.
+__device__ __forceinline__ int64_t counter_at_launch(const int64_t* p) {
+  using ConstWord = const __attribute__((address_space(4))) int64_t;
+  return *reinterpret_cast<ConstWord*>(reinterpret_cast<uintptr_t>(p));
+}
+
 // A failure: the status word of the device tells the host, the broken word of the workspace tells every
 // wavefront that comes later (of this launch and of the launches behind it).
 __device__ __forceinline__ void raise_status(const KernelArgs& a, uint32_t bits, int lane) {
@@ -283,7 +293,9 @@ __device__ __forceinline__ UnitOffsets unit_offsets(const Stream& st, uint32_t f
 // ---------------------------------------------------------------------------
 // Part `part` of the a.parts wavefronts that send stream (s -> r, ch): it walks its slice of every run.
 // With kTeam the parts are the a.team wavefronts of this workgroup and share part 0's counters.
-template <int kAux, int kUnitsInFlight, bool kTeam = false>
+// kOddStats: the statistics rows are an odd number of floats (the combine's packed log-sum-exps); the exchange
+// kernel never sees such rows, and a compile-time switch keeps their loads out of its instruction stream.
+template <int kAux, int kUnitsInFlight, bool kTeam = false, bool kOddStats = false>
 __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, int ch, int part, int lane, int wave,
                                            TeamLds* lds = nullptr) {
   HELIX_MARK(wave, 0, false);
@@ -306,8 +318,8 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
   int64_t step = 0, tail = 0;
   uint64_t broken = 0;
   if (leader) {
-    step = *token;
-    tail = info[1];
+    step = counter_at_launch(token);
+    tail = counter_at_launch(&info[1]);
     broken = broken_at_launch(a);
   }
 
@@ -373,7 +385,7 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
           uint32_t U = U0 + i * kWaveLanes + lane;
           RunUnit d;
           UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < slice.end, &d);
-          if ((a.field1Bytes & 7) == 0) {
+          if (!kOddStats) {
             sa[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.a1, 0, kAuxNone);
             sb[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.b1, 0, kAuxNone);
           } else {
@@ -451,7 +463,7 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
   int64_t step = 0, head = 0;
   bool broken = false;
   if (leader) {
-    step = *mine;
+    step = counter_at_launch(mine);
     head = ld_counter(token);
     broken = broken_at_launch(a) != 0;
     if (kTeam && lane == 0) *reinterpret_cast<volatile int*>(&lds->bad) = 0;  // ahead of the team's first barrier
@@ -513,25 +525,16 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
         uint32_t off = U < passEnd ? entryOffset + U * kUnitBytes : kOutOfRange;
         v[i] = __builtin_amdgcn_raw_buffer_load_b128(st.fifo, off, 0, kAux);
       }
-      // every line carries its flag in the very load that brought its last unit
+      // Loads return in the order they were issued and the stores of access i need nothing but the load of access
+      // i (the realigned variant: and of i + 1), so every store goes out as soon as its own lines are back, while
+      // the later ones are still in flight. Every line carries its flag in the very load that brought its last
+      // unit; the flags are compared on the way, without a branch, and looked at once the pass is stored.
+      if (U0 == slice.begin && firstMsg == 0) HELIX_MARK(wave, 1, false);
       bool flagsAgree = true;
 #pragma unroll
       for (int i = 0; i < kUnitsInFlight; ++i) {
         uint32_t U = U0 + i * kWaveLanes + lane;
         flagsAgree &= U >= passEnd || (U & 7u) != 7u || (v[i].z == stepLo && v[i].w == stepHi);
-      }
-      if (__ballot(!flagsAgree) != 0ull) {
-        raise_status(a, kStatusInternal, lane);
-        if (!kTeam) return;
-        // a wavefront of a team stays with its team to the next barrier, where the leader learns of it; it
-        // stores nothing any more, and the workspace is marked broken
-        if (!corrupt) team_report_bad(lds, lane);
-        corrupt = true;
-      }
-      if (U0 == slice.begin && firstMsg == 0) HELIX_MARK(wave, 1, false);
-#pragma unroll
-      for (int i = 0; i < kUnitsInFlight; ++i) {
-        uint32_t U = U0 + i * kWaveLanes + lane;
         RunUnit d;
         UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < passEnd && !(kTeam && corrupt), &d);
         u32x2 wa = {v[i].x, v[i].y};
@@ -590,6 +593,15 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
           __builtin_amdgcn_raw_buffer_store_b64(wb, st.field1, o.b1, 0, kAuxNone);
         }
       }
+      if (__ballot(!flagsAgree) != 0ull) {
+        // a line of this pass did not carry the step: the pass went out as it came, nothing goes out after it
+        raise_status(a, kStatusInternal, lane);
+        if (!kTeam) return;
+        // a wavefront of a team stays with its team to the next barrier, where the leader learns of it; it
+        // stores nothing any more, and the workspace is marked broken
+        if (!corrupt) team_report_bad(lds, lane);
+        corrupt = true;
+      }
     }
   }
   HELIX_MARK(wave, 2, false);
@@ -603,15 +615,15 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
 }
 
 // The one wave-uniform branch on the units-in-flight count of the launch.
-template <int kAux>
+template <int kAux, bool kOddStats>
 __device__ __forceinline__ void run_sender_any(const KernelArgs& a, int s, int r, int ch, int part, int lane, int wave) {
   switch (a.unitsInFlight) {
-    case 1: run_sender<kAux, 1>(a, s, r, ch, part, lane, wave); break;
-    case 2: run_sender<kAux, 2>(a, s, r, ch, part, lane, wave); break;
-    case 3: run_sender<kAux, 3>(a, s, r, ch, part, lane, wave); break;
-    case 4: run_sender<kAux, 4>(a, s, r, ch, part, lane, wave); break;
-    case 5: run_sender<kAux, 5>(a, s, r, ch, part, lane, wave); break;
-    default: run_sender<kAux, kMaxUnitsInFlight>(a, s, r, ch, part, lane, wave); break;
+    case 1: run_sender<kAux, 1, false, kOddStats>(a, s, r, ch, part, lane, wave); break;
+    case 2: run_sender<kAux, 2, false, kOddStats>(a, s, r, ch, part, lane, wave); break;
+    case 3: run_sender<kAux, 3, false, kOddStats>(a, s, r, ch, part, lane, wave); break;
+    case 4: run_sender<kAux, 4, false, kOddStats>(a, s, r, ch, part, lane, wave); break;
+    case 5: run_sender<kAux, 5, false, kOddStats>(a, s, r, ch, part, lane, wave); break;
+    default: run_sender<kAux, kMaxUnitsInFlight, false, kOddStats>(a, s, r, ch, part, lane, wave); break;
   }
 }
 // Wavefront w of a launch: sender wavefronts come first in dispatch order so
@@ -972,7 +984,10 @@ __global__ __launch_bounds__(kMaxCombineParts * kWaveLanes) HELIX_WAVES_PER_SIMD
     if (w >= senderStreams) return;
     const int t = static_cast<int>(fast_div_by(static_cast<uint32_t>(w), a.byCp));
     const int localIndex = static_cast<int>(fast_div_by(static_cast<uint32_t>(t), a.byChannels));
-    run_sender_any<kAuxSc1>(a, a.rankBegin + localIndex, w - t * a.cpSize, t - localIndex * a.runChannels, 0, lane, w);
+    if ((a.field1Bytes & 7) == 0)
+      run_sender_any<kAuxSc1, false>(a, a.rankBegin + localIndex, w - t * a.cpSize, t - localIndex * a.runChannels, 0, lane, w);
+    else
+      run_sender_any<kAuxSc1, true>(a, a.rankBegin + localIndex, w - t * a.cpSize, t - localIndex * a.runChannels, 0, lane, w);
     return;
   }
   b -= sendBlocks;

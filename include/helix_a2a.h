@@ -252,10 +252,10 @@ int helix_a2a_device_status(uint32_t* status, void* stream);
  * -- the rest of the launch and every launch queued behind it -- writes nothing
  * and raises HELIX_A2A_STATUS_BROKEN_WORKSPACE, so the output tensors of
  * such an exchange keep whatever they held before; the FIFO counters are no
- * longer consistent. (Where the wavefronts of a workgroup walk a run as a team,
- * the one that met the corrupt line stores nothing from that pass on, its
- * team-mates finish the pass they are in, and the stream's counters stay where
- * they were.) helix_a2a_init_workspace on row 0 (with the other rows)
+ * longer consistent. (The pass of at most 6 KiB in which a wavefront meets a
+ * corrupt line goes out as it came; the wavefront stores nothing after it.
+ * Where the wavefronts of a workgroup walk a run as a team, the others finish
+ * the pass they are in, and the stream's counters stay where they were.) helix_a2a_init_workspace on row 0 (with the other rows)
  * makes the workspace usable again. The calls themselves return at launch, so
  * a caller learns of a failure from helix_a2a_device_status, or at once in
  * checked mode:

@@ -769,10 +769,9 @@ def test_corrupt_line_is_reported(hx, ops, teams, unchecked):
         status = ops.device_status()
         assert status & ops.STATUS_INTERNAL, status
         if teams:
-            # 3 messages of 513 pieces on one channel: a run of 103 lines walked by 7 wavefronts, 16 lines each.
-            # The wavefront that owns lines 32..47 (run pieces 480..719: the end of message 0 and pieces 0..206
-            # of message 1) stores nothing; its team-mates store their slices; the stream's counters stay put
-            assert bool((out_o[1][1, 0, :800].view(torch.int16) == 0).all())
+            # 3 messages of 513 pieces on one channel: a run of 103 lines walked by 7 wavefronts, 16 lines each,
+            # one pass per wavefront. The wavefront that owns lines 32..47 stores its pass as it came and reports;
+            # its team-mates store their slices; the stream's counters stay put
             assert bits_equal(out_o[1][2, 0], o[0][2, 1])
             max_ch = _max_channels(cp)
             receiver_info = (512 * 1024 * cp * max_ch + 256 * cp * max_ch) // 8
