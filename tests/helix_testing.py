@@ -59,7 +59,8 @@ class HostModel:
     """ctypes front end of tests/host_model (the bounds-checked CPU walk-through of the GPU wave programs)."""
 
     def __init__(self) -> None:
-        if not HOST_MODEL_LIB.exists():
+        sources = [HOST_MODEL_DIR / "helix_host_model.cpp", *(ROOT / "helix-a2a_amd" / "csrc").glob("*.hpp")]
+        if not HOST_MODEL_LIB.exists() or HOST_MODEL_LIB.stat().st_mtime < max(f.stat().st_mtime for f in sources):
             build_host_model()
         lib = ctypes.CDLL(str(HOST_MODEL_LIB))
         lib.hm_alltoall.argtypes = [ctypes.POINTER(_Params)] + [ctypes.c_int] * 5
