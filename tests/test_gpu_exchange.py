@@ -301,6 +301,51 @@ def test_ragged_shapes(hx, ops, cp, entries, x, s):
         assert outs_o[0].shape == ins_o[0].shape
 
 
+def _seeded_cases(count, seed):
+    """(cp, entries, x, s, channels, team_units, units_per_wavefront) drawn from one seed: ragged sizes, every
+    rank count up to eight and sixteen, channel counts from one to all the layout provides, every sharing rule."""
+    import random
+    rng = random.Random(seed)
+    cases = []
+    while len(cases) < count:
+        cp = rng.choice([1, 2, 3, 4, 5, 6, 7, 8, 16])
+        x = 8 * rng.choice([1, 2, 3, 5, 8, 17, 32, 33, 64, 100, 128, 255, 256, 512, 1000, 2048])
+        s = rng.choice([2, 2, 2, 4, 6, 8, 14, 16, 32, 62])
+        entries = rng.choice([1, 2, 3, 7, 16, 33, 64, 100, 129, 256, 300])
+        if cp * cp * entries * (2 * x + 4 * s) > 96 << 20:   # keeps the whole test within seconds
+            continue
+        channels = rng.choice([0, 0, 1, 2, 3, 5, 8, 16, 31, 64, 128])
+        cases.append((cp, entries, x, s, channels, rng.choice([-1, -1, 0, 2, 6]), rng.choice([-1, -1, 0, 3])))
+    return cases
+
+
+def test_seeded_random_shapes_on_shared_workspaces(hx, ops):
+    # sixty exchanges of unrelated shapes, one after the other on the workspaces of their rank counts: whatever
+    # a launch leaves in the counters and the FIFO slots is what the next one, with another placement of its
+    # runs, starts from; every result bit-exact against the closed form
+    try:
+        for i, (cp, entries, x, s, channels, team_units, units) in enumerate(_seeded_cases(60, 20240607)):
+            ws = get_workspace(hx, cp)
+            channels = min(channels, _max_channels(cp))
+            g = torch.Generator().manual_seed(7000 + i)
+            ins_o = [torch.randint(-32768, 32767, (entries, cp, x), generator=g, dtype=torch.int16).view(torch.bfloat16).cuda()
+                     for _ in range(cp)]
+            ins_s = [torch.randint(-2**31, 2**31 - 1, (entries, cp, s), generator=g, dtype=torch.int32).view(torch.float32).cuda()
+                     for _ in range(cp)]
+            ops.set_team_units(team_units)
+            ops.set_units_per_wavefront(units)
+            outs_o, outs_s = hx.alltoall_loopback(ins_o, ins_s, ws, channel_count=channels)
+            torch.cuda.synchronize()
+            assert ops.device_status() == 0, (i, cp, entries, x, s, channels, team_units, units)
+            want_o, want_s = expected_on_device(ins_o), expected_on_device(ins_s)
+            for r in range(cp):
+                assert bits_equal(outs_o[r], want_o[r]) and bits_equal(outs_s[r], want_s[r]), \
+                    (i, r, cp, entries, x, s, channels, team_units, units)
+    finally:
+        ops.set_team_units(-1)
+        ops.set_units_per_wavefront(-1)
+
+
 @pytest.mark.parametrize("entries,units_in_flight", [(1, 1), (3, 2), (5, 3), (7, 4), (9, 5), (11, 6), (12, 4), (33, 6)])
 def test_every_units_in_flight_variant(hx, ops, entries, units_in_flight):
     # one channel, 520-byte messages (65 pieces): the run of `entries` messages, packed piece by piece into
