@@ -37,6 +37,7 @@ struct KernelArgs {
   int doSend, doRecv;
   int unitsInFlight;        // units_in_flight_for_run(largest run of the launch), 1..kMaxUnitsInFlight
   int alignedStores;        // receivers realign payload to 16-byte stores: set when runs take several passes
+  int longRuns;             // the largest run of the launch takes several passes (combine kernel: receivers first look at the senders' counters through the scalar cache)
   int parts;                // wavefronts that share one stream's runs (per direction), 1..kMaxStreamParts
   int team;                 // exchange kernel: wavefronts of a workgroup that walk one stream's run together (parts == 1), 1..kMaxTeamWavefronts
   // Worked out by the launch functions from the fields above, so that no wavefront divides:
