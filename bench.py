@@ -40,12 +40,12 @@ MIN_ROOFLINE_STEPS = 200
 # <kernel>_<workload>.md hold the runs these come from. These counters sit between L2 and fabric:
 # they do not tell whether the memory-side cache or DRAM served a request.
 MEASURED_TRAFFIC_BYTES = {
-    ("helix_exchange_kernel", "c3", 128): 151_042_589,   # profiles/helix_exchange_kernel_c3.md
-    ("helix_exchange_kernel", "c4", 128): 566_976_087,   # profiles/helix_exchange_kernel_c4.md
-    ("helix_exchange_kernel", "c5a", 64): 588_616_310,   # profiles/helix_exchange_kernel_c5a.md
-    ("helix_combine_kernel", "c3", 128): 118_817_682,   # profiles/helix_combine_kernel_c3.md
-    ("helix_combine_kernel", "c4", 128): 451_089_053,   # profiles/helix_combine_kernel_c4.md
-    ("helix_combine_kernel", "c5a", 64): 464_922_527,   # profiles/helix_combine_kernel_c5a.md
+    ("helix_exchange_kernel", "c3", 128): 151_088_104,   # profiles/helix_exchange_kernel_c3.md
+    ("helix_exchange_kernel", "c4", 128): 567_478_447,   # profiles/helix_exchange_kernel_c4.md
+    ("helix_exchange_kernel", "c5a", 64): 588_734_486,   # profiles/helix_exchange_kernel_c5a.md
+    ("helix_combine_kernel", "c3", 128): 118_759_652,   # profiles/helix_combine_kernel_c3.md
+    ("helix_combine_kernel", "c4", 128): 450_300_841,   # profiles/helix_combine_kernel_c4.md
+    ("helix_combine_kernel", "c5a", 64): 462_194_517,   # profiles/helix_combine_kernel_c5a.md
 }
 
 
