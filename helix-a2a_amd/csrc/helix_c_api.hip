@@ -326,6 +326,7 @@ int build_plan(const helix_a2a_params_t* ranks, int count, bool exchangeOutputs,
   a.recvBytes0 = static_cast<uint32_t>(rows * a.recvStride0);
   a.recvBytes1 = static_cast<uint32_t>(rows * a.recvStride1);
   a.npMagic = div_magic(static_cast<uint32_t>(sh.np));
+  a.nsMagic = div_magic(static_cast<uint32_t>(sh.np - sh.np0));
   a.rankBegin = p0.cp_rank;
   a.rankCount = count;
   a.spinLimitTicks = g_spinLimitUs.load() * 100ull;

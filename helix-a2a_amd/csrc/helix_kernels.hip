@@ -224,7 +224,7 @@ __device__ __forceinline__ void fetch_scalars_up_front(const KernelArgs& a) {
   asm volatile("" ::"s"(a.workspace), "s"(a.rowStrideBytes), "s"(a.cpSize), "s"(a.maxChannels), "s"(a.runChannels),
                "s"(a.entryBegin), "s"(a.field0Bytes), "s"(a.field1Bytes), "s"(a.sendStride0), "s"(a.sendStride1),
                "s"(a.recvStride0), "s"(a.recvStride1), "s"(a.sendBytes0), "s"(a.sendBytes1), "s"(a.recvBytes0),
-               "s"(a.recvBytes1), "s"(a.npMagic), "s"(a.rankBegin), "s"(a.rankCount), "s"(a.doSend), "s"(a.doRecv));
+               "s"(a.recvBytes1), "s"(a.npMagic), "s"(a.nsMagic), "s"(a.rankBegin), "s"(a.rankCount), "s"(a.doSend), "s"(a.doRecv));
   asm volatile("" ::"s"(a.parts), "s"(a.team), "s"(a.np0), "s"(a.np), "s"(a.msgsPerEntry), "s"(a.baseMsgs),
                "s"(a.extraChannels), "s"(a.byParts.magic), "s"(a.byParts.shift), "s"(a.byTeam.magic), "s"(a.byTeam.shift),
                "s"(a.byCp.magic), "s"(a.byCp.shift), "s"(a.byChannels.magic), "s"(a.byChannels.shift), "s"(a.sendBlocks), "s"(a.wavesPerBlock), "s"(a.dirBlocks), "s"(a.xcdGroup),
@@ -240,6 +240,7 @@ struct Stream {
   uint32_t firstRow;              // row of the stream's first message of this launch
   uint32_t rowStep;               // rows between consecutive messages of the stream
   uint32_t np0, np, npMagic;       // pieces of field 0, of a message, div_magic(np)
+  uint32_t ns, nsMagic;           // statistics pieces of a message (np - np0), div_magic(ns)
   int msgs;                       // messages of the stream in this launch
   int msgsPerEntry;
 };
@@ -248,6 +249,8 @@ __device__ __forceinline__ void setup_stream(Stream& st, const KernelArgs& a, in
   st.np0 = static_cast<uint32_t>(a.np0);
   st.np = static_cast<uint32_t>(a.np);
   st.npMagic = a.npMagic;
+  st.ns = st.np - st.np0;
+  st.nsMagic = a.nsMagic;
   st.msgsPerEntry = a.msgsPerEntry;
   st.msgs = a.baseMsgs + (ch < a.extraChannels ? 1 : 0);  // stream_msg_count(a.entryBegin, a.entryEnd, ch, a.runChannels)
   st.firstRow = static_cast<uint32_t>(a.entryBegin + ch) * a.cpSize + peer;
@@ -364,6 +367,36 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
       return step >= 0;
     };
     for (uint32_t U0 = slice.begin; U0 < slice.end; U0 += kUnitsInFlight * kWaveLanes) {
+      // Statistics first: the statistics pieces of the whole pass in one load (two, beyond 64 pieces), lane j
+      // taking the j-th of them in run order; the lanes that store them pick them up below. One load per wave
+      // access that touches the end of a message, a few live lanes each, cost a sender as much as its payload
+      // loads did. Loads return in the order they were issued, so with these first every store below waits for
+      // the payload of its own access only.
+      const uint32_t passFirst = (U0 / kUnitsPerLine) * kPiecesPerLine;
+      uint32_t passEnd = passFirst + kUnitsInFlight * (kWaveLanes / kUnitsPerLine) * kPiecesPerLine;
+      passEnd = min(passEnd, min(static_cast<uint32_t>(runMsgs) * st.np, (slice.end / kUnitsPerLine) * kPiecesPerLine));
+      const uint32_t ordFirst = stats_ordinal_at(passFirst, st.np, st.np0, st.npMagic);
+      const uint32_t ordEnd = passEnd > passFirst ? stats_ordinal_at(passEnd, st.np, st.np0, st.npMagic) : ordFirst;
+      u32x2 gathered[kStatsGathers];
+#pragma unroll
+      for (int c = 0; c < kStatsGathers; ++c) {
+        gathered[c] = u32x2{0u, 0u};
+        if (ordFirst + c * kWaveLanes < ordEnd) {  // wave-uniform
+          const uint32_t ord = ordFirst + c * kWaveLanes + lane;
+          const uint32_t m = div_by_magic(ord, st.nsMagic);
+          const uint32_t index = ord - m * st.ns;
+          const uint32_t row = st.firstRow + (firstMsg + m) * st.rowStep;
+          const uint32_t off = ord < ordEnd ? row * st.stride1 + index * kPieceBytes : kOutOfRange;
+          if (!kOddStats) {
+            gathered[c] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, off, 0, kAuxNone);
+          } else {
+            // rows of an odd number of floats (one log-sum-exp per head): 4-byte aligned, and the upper
+            // half of a row's last piece is not part of the row -- it travels as zero
+            gathered[c].x = __builtin_amdgcn_raw_buffer_load_b32(st.field1, off, 0, kAuxNone);
+            gathered[c].y = __builtin_amdgcn_raw_buffer_load_b32(st.field1, (off != kOutOfRange && index + 1u != st.ns) ? off + 4u : kOutOfRange, 0, kAuxNone);
+          }
+        }
+      }
       u32x2 wa[kUnitsInFlight], wb[kUnitsInFlight];
       unsigned long long needField1[kUnitsInFlight];  // wave-uniform: lanes of access i that hold statistics pieces
 #pragma unroll
@@ -374,51 +407,46 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
         wb[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field0, o.b0, 0, kAuxNone);
         needField1[i] = __ballot((o.a1 != kOutOfRange) | (o.b1 != kOutOfRange));
       }
-      // Statistics are the last few pieces of a message: only the accesses that
-      // cover the end of a message read the second tensor at all.
-      u32x2 sa[kUnitsInFlight], sb[kUnitsInFlight];
-#pragma unroll
-      for (int i = 0; i < kUnitsInFlight; ++i) {
-        sa[i] = u32x2{0u, 0u};
-        sb[i] = u32x2{0u, 0u};
-        if (needField1[i] != 0ull) {
-          uint32_t U = U0 + i * kWaveLanes + lane;
-          RunUnit d;
-          UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < slice.end, &d);
-          if (!kOddStats) {
-            sa[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.a1, 0, kAuxNone);
-            sb[i] = __builtin_amdgcn_raw_buffer_load_b64(st.field1, o.b1, 0, kAuxNone);
-          } else {
-            // rows of an odd number of floats (one log-sum-exp per head): 4-byte aligned, and the upper
-            // half of a row's last piece is not part of the row -- it travels as zero
-            const uint32_t lastPiece = st.np - 1u;
-            const uint32_t aHi = (o.a1 != kOutOfRange && d.pieceA != lastPiece) ? o.a1 + 4u : kOutOfRange;
-            const uint32_t bHi = (o.b1 != kOutOfRange && d.pieceB != lastPiece) ? o.b1 + 4u : kOutOfRange;
-            sa[i].x = __builtin_amdgcn_raw_buffer_load_b32(st.field1, o.a1, 0, kAuxNone);
-            sa[i].y = __builtin_amdgcn_raw_buffer_load_b32(st.field1, aHi, 0, kAuxNone);
-            sb[i].x = __builtin_amdgcn_raw_buffer_load_b32(st.field1, o.b1, 0, kAuxNone);
-            sb[i].y = __builtin_amdgcn_raw_buffer_load_b32(st.field1, bHi, 0, kAuxNone);
-          }
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < kUnitsInFlight; ++i) {
-        wa[i] |= sa[i];
-        wb[i] |= sb[i];
-      }
-      if (!opened && !open_entry()) return;
+      // A wavefront that gives up here still runs through the stores of the pass, every lane out of range, and
+      // leaves after them: an exit between the loads and the stores leaves through the end of this loop in the
+      // compiled code, which then counts the loads as still in flight when the next pass starts and makes every
+      // pass wait for registers that are long back.
+      const bool open = opened || open_entry();
       if (U0 == slice.begin && firstMsg == 0) HELIX_MARK(wave, 1, true);
       const uint32_t entryOffset = (static_cast<uint32_t>(step) & a.positionMask) * a.positionBytes;
       const uint32_t stepLo = static_cast<uint32_t>(step);
       const uint32_t stepHi = static_cast<uint32_t>(static_cast<uint64_t>(step) >> 32);
+      // the statistics piece with ordinal `ord`, from the lane that loaded it
+      auto statistics_piece = [&](uint32_t ord) -> u32x2 {
+        const uint32_t rel = ord - ordFirst;
+        const int from = static_cast<int>((rel & (kWaveLanes - 1)) * 4u);
+        u32x2 v = {static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(gathered[0].x))),
+                   static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(gathered[0].y)))};
+        if (ordFirst + kWaveLanes < ordEnd) {  // wave-uniform: a second load was needed
+          const u32x2 w = {static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(gathered[1].x))),
+                           static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(gathered[1].y)))};
+          if (rel >= static_cast<uint32_t>(kWaveLanes)) v = w;
+        }
+        return v;
+      };
 #pragma unroll
       for (int i = 0; i < kUnitsInFlight; ++i) {
         uint32_t U = U0 + i * kWaveLanes + lane;
         bool flag = (U & 7u) == 7u;
-        u32x4 v = {wa[i].x, wa[i].y, flag ? stepLo : wb[i].x, flag ? stepHi : wb[i].y};
-        uint32_t off = U < slice.end ? entryOffset + U * kUnitBytes : kOutOfRange;
+        u32x2 pa = wa[i], pb = wb[i];
+        if (needField1[i] != 0ull) {  // a piece comes from one of the two tensors; the payload load gave zeros elsewhere
+          RunUnit d;
+          UnitOffsets o = unit_offsets(st, firstMsg, runMsgs, U, U < slice.end, &d);
+          const u32x2 sa = statistics_piece(d.msgA * st.ns + (d.pieceA - st.np0));
+          const u32x2 sb = statistics_piece(d.msgB * st.ns + (d.pieceB - st.np0));
+          if (o.a1 != kOutOfRange) pa = sa;
+          if (o.b1 != kOutOfRange) pb = sb;
+        }
+        u32x4 v = {pa.x, pa.y, flag ? stepLo : pb.x, flag ? stepHi : pb.y};
+        uint32_t off = (open && U < slice.end) ? entryOffset + U * kUnitBytes : kOutOfRange;
         __builtin_amdgcn_raw_buffer_store_b128(v, st.fifo, off, 0, kAux);
       }
+      if (!open) return;
     }
     if (!opened && !open_entry()) return;  // nothing of this run falls to this part: the step still counts
   }
@@ -1074,7 +1102,8 @@ static int xcd_group_for(int wavesPerPeerSet, int wavesPerBlock, int streamsPerB
   return group;
 }
 
-// The fields of the argument block that follow from the others (see KernelArgs); a.parts and a.team are set.
+// The fields of the argument block that follow from the others (see KernelArgs); a.parts, a.team and
+// a.unitsInFlight are set.
 static void set_launch_constants(KernelArgs& a) {
   const MsgShape sh = make_msg_shape(a.field0Bytes, a.field1Bytes);
   a.np0 = sh.np0;
@@ -1093,6 +1122,9 @@ static void set_launch_constants(KernelArgs& a) {
   a.byTeam = fast_div(static_cast<uint32_t>(a.team));
   a.byCp = fast_div(static_cast<uint32_t>(a.cpSize));
   a.byChannels = fast_div(static_cast<uint32_t>(a.runChannels));
+  // messages that are mostly statistics: passes short enough for the senders' gather (a.unitsInFlight is set)
+  const int forStatistics = max_units_in_flight_for_statistics(a.np, a.np0);
+  if (a.unitsInFlight > forStatistics) a.unitsInFlight = forStatistics;
 }
 
 hipError_t launch_exchange(const KernelArgs& args, int unitsPerPart, int maxParts, int teamUnits, hipStream_t stream) {

@@ -33,6 +33,7 @@ struct KernelArgs {
   uint32_t sendBytes0, sendBytes1;  // extent of each tensor (< 2 GiB), the range of its buffer descriptor
   uint32_t recvBytes0, recvBytes1;
   uint32_t npMagic;                 // div_magic(pieces per message)
+  uint32_t nsMagic;                 // div_magic(statistics pieces per message)
   int rankBegin, rankCount;
   int doSend, doRecv;
   int unitsInFlight;        // units_in_flight_for_run(largest run of the launch), 1..kMaxUnitsInFlight

@@ -243,6 +243,17 @@ HELIX_HD RunUnit decode_run_unit(uint32_t U, uint32_t np, uint32_t npMagic) {
   return d;
 }
 
+// ---- the statistics pieces of a run, counted ----------------------------------
+// Message m of a run holds its statistics in its last ns = np - np0 pieces; its i-th statistics piece is the
+// run's statistics piece number ("ordinal") m * ns + i. A sender fetches the statistics pieces of one pass with
+// one load -- lane j takes the j-th of them -- and hands every piece to the lane that stores it, instead of one
+// load of a few live lanes per wave access that touches the end of a message.
+// Statistics pieces of the run that sit before run piece P:
+HELIX_HD uint32_t stats_ordinal_at(uint32_t P, uint32_t np, uint32_t np0, uint32_t npMagic) {
+  const uint32_t m = div_by_magic(P, npMagic);
+  const uint32_t q = P - m * np;
+  return m * (np - np0) + (q > np0 ? q - np0 : 0u);
+}
 // Head index of payload piece p when a head spans `piecesPerHead` pieces (head_dim * 2 bytes / 8).
 HELIX_HD uint32_t head_div_magic(uint32_t piecesPerHead) { return div_magic(piecesPerHead); }
 HELIX_HD uint32_t head_of_piece(uint32_t p, uint32_t magic) { return div_by_magic(p, magic); }
@@ -266,6 +277,22 @@ HELIX_HD int units_in_flight_for_run(long runUnits) {
   long passes = (perLane + kMaxUnitsInFlight - 1) / kMaxUnitsInFlight;
   return static_cast<int>((perLane + passes - 1) / passes);
 }
+
+// A pass of `unitsInFlight` units per lane covers unitsInFlight * 120 consecutive pieces of the run; a sender
+// gathers its statistics pieces in at most kStatsGathers loads of 64. Whatever the shape, a pass of one unit
+// per lane (120 pieces) fits; launches whose messages are mostly statistics take fewer units per pass.
+constexpr int kStatsGathers = 2;
+HELIX_HD int max_units_in_flight_for_statistics(int np, int np0) {
+  const int ns = np - np0;
+  for (int k = kMaxUnitsInFlight; k > 1; --k) {
+    const int pieces = k * (kWaveLanes / kUnitsPerLine) * kPiecesPerLine;
+    int most = (pieces / np + 2) * ns;   // message ends a pass can touch, all of their statistics
+    if (most > pieces) most = pieces;
+    if (most <= kStatsGathers * kWaveLanes) return k;
+  }
+  return 1;
+}
+
 
 
 // ---- runs shared by several wavefronts ---------------------------------------

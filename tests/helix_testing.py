@@ -71,6 +71,10 @@ class HostModel:
         lib.hm_fifo_positions.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_long, ctypes.c_int]
         lib.hm_fifo_positions.restype = ctypes.c_int
         lib.hm_stream_fifo_offset.restype = ctypes.c_uint64
+        lib.hm_stats_ordinal_at.argtypes = [ctypes.c_uint32, ctypes.c_int, ctypes.c_int]
+        lib.hm_stats_ordinal_at.restype = ctypes.c_uint32
+        lib.hm_max_units_for_statistics.argtypes = [ctypes.c_int, ctypes.c_int]
+        lib.hm_max_units_for_statistics.restype = ctypes.c_int
         lib.hm_packed_slot_bytes.argtypes = [ctypes.c_long]
         lib.hm_packed_slot_bytes.restype = ctypes.c_uint32
         for name in ("hm_sender_info_offset", "hm_receiver_info_offset"):

@@ -130,18 +130,53 @@ void run_sender(Ctx& c, int s, int r, int ch, int part) {
     // tighter than the GPU's descriptor: every access must stay inside the stream's slot of this step's quarter
     Extent fifoExt{fifo + entryOffset, c.slotBytes};
     if (!c.chk.ok(c.fifoRegion(r), fifoExt.base, c.slotBytes, "fifo slot")) return;
-    for (uint32_t U = slice.begin; U < slice.end; ++U) {  // every lane of every wave access
-      UnitOffsets o = unit_offsets(c, firstRow, rowStep, p.send_fields[0].stride_bytes, p.send_fields[1].stride_bytes,
-                                   firstMsg, runMsgs, U);
-      uint64_t words[2] = {0, 0};
-      const uint32_t offs0[2] = {o.a0, o.b0}, offs1[2] = {o.a1, o.b1};
-      for (int k = 0; k < 2; ++k) {
-        if (offs0[k] != kNone && c.chk.ok(e0, e0.base + offs0[k], 8, "send field 0")) memcpy(&words[k], e0.base + offs0[k], 8);
-        if (offs1[k] != kNone && c.chk.ok(e1, e1.base + offs1[k], 8, "send field 1")) memcpy(&words[k], e1.base + offs1[k], 8);
+    // one pass = unitsInFlight accesses of 64 lanes. The statistics pieces of the pass are gathered first, lane j
+    // of gather g taking the pass's statistics piece number g * 64 + j in run order; the lanes that store a
+    // statistics piece take it from there.
+    const uint32_t np = static_cast<uint32_t>(c.sh.np), np0 = static_cast<uint32_t>(c.sh.np0), ns = np - np0;
+    const uint32_t passUnits = static_cast<uint32_t>(c.unitsInFlight) * kWaveLanes;
+    for (uint32_t U0 = slice.begin; U0 < slice.end; U0 += passUnits) {
+      const uint32_t passFirst = (U0 / kUnitsPerLine) * kPiecesPerLine;
+      uint32_t passEnd = passFirst + static_cast<uint32_t>(c.unitsInFlight) * (kWaveLanes / kUnitsPerLine) * kPiecesPerLine;
+      if (passEnd > static_cast<uint32_t>(runMsgs) * np) passEnd = static_cast<uint32_t>(runMsgs) * np;
+      if (passEnd > (slice.end / kUnitsPerLine) * kPiecesPerLine) passEnd = (slice.end / kUnitsPerLine) * kPiecesPerLine;
+      const uint32_t ordFirst = stats_ordinal_at(passFirst, np, np0, div_magic(np));
+      const uint32_t ordEnd = passEnd > passFirst ? stats_ordinal_at(passEnd, np, np0, div_magic(np)) : ordFirst;
+      if (ordEnd - ordFirst > static_cast<uint32_t>(kStatsGathers * kWaveLanes)) {
+        c.chk.violations++;
+        snprintf(c.chk.first, sizeof(c.chk.first), "sender %d->%d ch %d: %u statistics pieces in one pass", s, r, ch, ordEnd - ordFirst);
+        return;
       }
-      if (o.flag) words[1] = static_cast<uint64_t>(step);
-      uint8_t* dst = fifo + entryOffset + U * kUnitBytes;
-      if (c.chk.ok(fifoExt, dst, 16, "fifo store")) memcpy(dst, words, 16);
+      uint64_t gathered[kStatsGathers * kWaveLanes] = {0};
+      for (uint32_t ord = ordFirst; ord < ordEnd; ++ord) {
+        const uint32_t m = div_by_magic(ord, div_magic(ns));
+        const uint32_t index = ord - m * ns;
+        const uint32_t off = (firstRow + (firstMsg + m) * rowStep) * p.send_fields[1].stride_bytes + index * kPieceBytes;
+        if (c.chk.ok(e1, e1.base + off, 8, "send field 1")) memcpy(&gathered[ord - ordFirst], e1.base + off, 8);
+      }
+      for (uint32_t U = U0; U < U0 + passUnits && U < slice.end; ++U) {  // every lane of every wave access
+        RunUnit d;
+        UnitOffsets o = unit_offsets(c, firstRow, rowStep, p.send_fields[0].stride_bytes, p.send_fields[1].stride_bytes,
+                                     firstMsg, runMsgs, U, &d);
+        uint64_t words[2] = {0, 0};
+        const uint32_t offs0[2] = {o.a0, o.b0}, offs1[2] = {o.a1, o.b1};
+        const uint32_t ords[2] = {d.msgA * ns + (d.pieceA - np0), d.msgB * ns + (d.pieceB - np0)};
+        for (int k = 0; k < 2; ++k) {
+          if (offs0[k] != kNone && c.chk.ok(e0, e0.base + offs0[k], 8, "send field 0")) memcpy(&words[k], e0.base + offs0[k], 8);
+          if (offs1[k] != kNone) {
+            if (ords[k] < ordFirst || ords[k] >= ordEnd) {
+              c.chk.violations++;
+              snprintf(c.chk.first, sizeof(c.chk.first), "sender %d->%d ch %d unit %u: statistics piece %u outside the pass's [%u, %u)",
+                       s, r, ch, U, ords[k], ordFirst, ordEnd);
+              return;
+            }
+            words[k] = gathered[ords[k] - ordFirst];
+          }
+        }
+        if (o.flag) words[1] = static_cast<uint64_t>(step);
+        uint8_t* dst = fifo + entryOffset + U * kUnitBytes;
+        if (c.chk.ok(fifoExt, dst, 16, "fifo store")) memcpy(dst, words, 16);
+      }
     }
   }
   *token = step + 1;
@@ -315,6 +350,7 @@ int hm_alltoall(const helix_a2a_params_t* per_rank, int cp, int cu_count, int ch
                                                   : split_for_run(maxRun, kMaxUnitsInFlight, auto_max_parts(cp, channels, cu_count));
       c.parts = split.parts;
       c.unitsInFlight = split.unitsInFlight;
+      if (c.unitsInFlight > max_units_in_flight_for_statistics(c.sh.np, c.sh.np0)) c.unitsInFlight = max_units_in_flight_for_statistics(c.sh.np, c.sh.np0);
       c.alignedStores = maxRun > static_cast<long>(kMaxUnitsInFlight) * kWaveLanes;
       const int msgsMax = stream_msg_count(c.entryBegin, c.entryEnd, 0, channels);
       c.positionMask = static_cast<uint32_t>(fifo_positions(exchange_lines_bytes(cp, channels, maxRun), entries_for_msgs(msgsMax, c.sh))) - 1u;
@@ -409,6 +445,10 @@ int hm_fast_div_mismatches(uint32_t d, int samples) {
   }
   return bad;
 }
+// Statistics pieces of a run of messages of np pieces (np0 of them payload) that sit before run piece P, and the
+// most units per lane a pass may take so that its statistics pieces fit the senders' gather.
+uint32_t hm_stats_ordinal_at(uint32_t P, int np, int np0) { return stats_ordinal_at(P, np, np0, div_magic(np)); }
+int hm_max_units_for_statistics(int np, int np0) { return max_units_in_flight_for_statistics(np, np0); }
 // lines of a run of `msgs` messages and messages per FIFO entry for a message of the two field sizes
 int hm_run_lines(int msgs, int field0_bytes, int field1_bytes) { return run_lines(msgs, make_msg_shape(field0_bytes, field1_bytes)); }
 int hm_msgs_per_entry(int field0_bytes, int field1_bytes) { return msgs_per_fifo_entry(make_msg_shape(field0_bytes, field1_bytes)); }

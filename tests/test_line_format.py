@@ -165,6 +165,30 @@ def test_piece_division_is_exact(host_model):
     assert [host_model.lib.hm_div(g, 33) for g in (0, 32, 33, 65, 66, 15359)] == [0, 0, 1, 1, 2, 465]
 
 
+def test_statistics_pieces_of_a_pass_fit_the_senders_gather(host_model):
+    # A sender fetches the statistics pieces of a pass -- K * 120 consecutive run pieces -- with at most two loads of
+    # 64 lanes, lane j taking the j-th of them. The count of statistics pieces before a run piece must be what
+    # counting them one by one gives, and the K the launch rule allows a shape must keep every pass within 128.
+    lib = host_model.lib
+    shapes = [(5, 2), (3, 2), (2, 1), (33, 32), (66, 64), (264, 256), (2064, 2048), (129, 128), (9, 8), (24, 8), (100, 3),
+              (15360, 15359), (15360, 15000), (300, 172), (7, 1), (120, 60), (121, 1)]
+    for np, np0 in shapes:
+        ns = np - np0
+        run_pieces = (15360 // np) * np
+        before = [0] * (run_pieces + 1)          # statistics pieces before run piece P, counted one by one
+        for P in range(run_pieces):
+            before[P + 1] = before[P] + (1 if P % np >= np0 else 0)
+        for P in list(range(0, min(run_pieces, 3 * np) + 1)) + list(range(0, run_pieces + 1, 120)) + [run_pieces]:
+            assert lib.hm_stats_ordinal_at(P, np, np0) == before[P], (np, np0, P)
+        k = lib.hm_max_units_for_statistics(np, np0)
+        assert 1 <= k <= 6
+        most = max(before[min(P + k * 120, run_pieces)] - before[P] for P in range(0, run_pieces, 120))
+        assert most <= 128, (np, np0, k, most)
+        if k < 6:   # the rule is not needlessly strict: one more unit per lane could overflow some shape's window bound
+            assert ((k + 1) * 120 // np + 2) * ns > 128
+    assert lib.hm_max_units_for_statistics(264, 256) == 6 and lib.hm_max_units_for_statistics(5, 2) == 1
+
+
 def test_messages_of_a_run_are_packed_piece_by_piece(host_model):
     # per-head layout of the benchmark shape: 264-byte messages = 33 pieces = 2.2 lines each. Five of them
     # are 165 pieces = exactly 11 lines, where one message per three lines would take 15.
