@@ -466,9 +466,10 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
 // part (that part's counter beyond the step: all its lines of the step are in memory), reads its slice
 // in passes of kUnitsInFlight units per lane and stores the payload. Line flags are still compared: one
 // that disagrees after the token means the workspace is corrupt.
+// `stage`: kStatsGathers * 64 pieces of LDS of this wavefront's own.
 template <int kAux, int kUnitsInFlight, bool kAlignedStores, bool kTeam = false>
 __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, int ch, int part, int lane, int wave,
-                                             TeamLds* lds = nullptr) {
+                                             u32x2* stage, TeamLds* lds = nullptr) {
   HELIX_MARK(wave, 0, false);
   const bool leader = !kTeam || part == 0;
   const int sliceCount = kTeam ? a.team : a.parts;
@@ -567,6 +568,12 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
       // unit; the flags are compared on the way, without a branch, and looked at once the pass is stored.
       if (U0 == slice.begin && firstMsg == 0) HELIX_MARK(wave, 1, false);
       bool flagsAgree = true;
+      // where the statistics pieces of the pass sit among those of the run (see run_sender)
+      const uint32_t piecesFirst = (U0 / kUnitsPerLine) * kPiecesPerLine;
+      const uint32_t piecesEnd = (kTeam && corrupt) ? piecesFirst
+                                                    : min((passEnd / kUnitsPerLine) * kPiecesPerLine, static_cast<uint32_t>(runMsgs) * st.np);
+      const uint32_t ordFirst = stats_ordinal_at(piecesFirst, st.np, st.np0, st.npMagic);
+      const uint32_t ordEnd = piecesEnd > piecesFirst ? stats_ordinal_at(piecesEnd, st.np, st.np0, st.npMagic) : ordFirst;
 #pragma unroll
       for (int i = 0; i < kUnitsInFlight; ++i) {
         uint32_t U = U0 + i * kWaveLanes + lane;
@@ -621,12 +628,38 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
           __builtin_amdgcn_raw_buffer_store_b64(wa, st.field0, o.a0, 0, kAuxNt);
           __builtin_amdgcn_raw_buffer_store_b64(wb, st.field0, o.b0, 0, kAuxNt);
         }
-        // statistics sit at the end of a message: few accesses touch the second tensor
+        // Statistics sit at the end of a message: few accesses hold pieces of the second tensor. Each such piece
+        // is put where the lane that stores it will look: slot "number of the piece among the statistics pieces of
+        // the pass" of this wavefront's staging row in LDS.
+        // (kernels of long runs only: where a run is one short pass, the trip through LDS at the end of the
+        // wavefront's only pass costs more than the few stores it saves -- c2 5.5 -> 5.9 us)
         if (__ballot((o.a1 != kOutOfRange) | (o.b1 != kOutOfRange)) != 0ull) {
+          if (kAlignedStores) {
+            if (o.a1 != kOutOfRange) stage[d.msgA * st.ns + (d.pieceA - st.np0) - ordFirst] = wa;
+            if (o.b1 != kOutOfRange) stage[d.msgB * st.ns + (d.pieceB - st.np0) - ordFirst] = wb;
+          } else {
+            // (no streaming hint: a statistics row can be as small as 8 bytes, and the rows of the
+            // cp senders share 64-byte sectors that the L2 should merge before they go to memory)
+            __builtin_amdgcn_raw_buffer_store_b64(wa, st.field1, o.a1, 0, kAuxNone);
+            __builtin_amdgcn_raw_buffer_store_b64(wb, st.field1, o.b1, 0, kAuxNone);
+          }
+        }
+      }
+      // The statistics pieces of the whole pass go out in one store (two, beyond 64 pieces), lane j taking the j-th
+      // of them in run order. One store of a few live lanes per wave access that touches the end of a message cost
+      // a receiver as much as its payload stores did.
+#pragma unroll
+      for (int c = 0; c < (kAlignedStores ? kStatsGathers : 0); ++c) {
+        if (ordFirst + c * kWaveLanes < ordEnd) {  // wave-uniform
+          const uint32_t ord = ordFirst + c * kWaveLanes + lane;
+          const uint32_t m = div_by_magic(ord, st.nsMagic);
+          const uint32_t index = ord - m * st.ns;
+          const uint32_t row = st.firstRow + (firstMsg + m) * st.rowStep;
+          const u32x2 piece = stage[c * kWaveLanes + lane];
           // (no streaming hint: a statistics row can be as small as 8 bytes, and the rows of the
           // cp senders share 64-byte sectors that the L2 should merge before they go to memory)
-          __builtin_amdgcn_raw_buffer_store_b64(wa, st.field1, o.a1, 0, kAuxNone);
-          __builtin_amdgcn_raw_buffer_store_b64(wb, st.field1, o.b1, 0, kAuxNone);
+          __builtin_amdgcn_raw_buffer_store_b64(piece, st.field1, ord < ordEnd ? row * st.stride1 + index * kPieceBytes : kOutOfRange,
+                                                0, kAuxNone);
         }
       }
       if (__ballot(!flagsAgree) != 0ull) {
@@ -673,6 +706,8 @@ __device__ __forceinline__ void run_sender_any(const KernelArgs& a, int s, int r
 template <int kUnitsInFlight, bool kAlignedStores, bool kTeam>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(kTeam ? 6 : 4, kTeam ? 6 : 4))) void helix_exchange_kernel(KernelArgs a) {
   __shared__ TeamLds teamLds;
+  // a row per wavefront, for the receivers of long runs
+  __shared__ u32x2 statisticsStage[!kAlignedStores ? 1 : kTeam ? kMaxTeamWavefronts : kMaxWavesPerBlock][kAlignedStores ? kStatsGathers * kWaveLanes : 1];
   fetch_scalars_up_front(a);
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWaveLanes);
   const int lane = static_cast<int>(threadIdx.x) % kWaveLanes;
@@ -694,7 +729,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(kTeam ? 6 
   if (isSender) {
     run_sender<kAuxSc1, kUnitsInFlight, kTeam>(a, local, peer, ch, part, lane, probe, &teamLds);
   } else {
-    run_receiver<kAuxSc1, kUnitsInFlight, kAlignedStores, kTeam>(a, local, peer, ch, part, lane, probe, &teamLds);
+    run_receiver<kAuxSc1, kUnitsInFlight, kAlignedStores, kTeam>(a, local, peer, ch, part, lane, probe, statisticsStage[kAlignedStores ? wave : 0], &teamLds);
   }
 }
 
@@ -1161,7 +1196,7 @@ hipError_t launch_exchange(const KernelArgs& args, int unitsPerPart, int maxPart
   // Wavefronts of a workgroup without teams are independent (no LDS, no barrier). Two per workgroup dispatch and
   // retire at the finest useful grain when wavefronts queue for slots; a launch that fits the device at once is
   // bound by how fast its workgroups are dispatched, and four per workgroup halve that (c2: 7.2 -> 6.6 us).
-  const int wpb = a.team > 1 ? a.team : waves <= kResidentWavefronts ? 4 : kWavesPerBlock;
+  const int wpb = a.team > 1 ? a.team : waves <= kResidentWavefronts ? kMaxWavesPerBlock : kWavesPerBlock;
   const int perDirection = waves / directions;
   a.dirBlocks = a.team > 1 ? perDirection : (perDirection + wpb - 1) / wpb;
   // (launches with teams stay as dispatched: regrouped, c4 in the per-head layout took 0.7 % longer)

@@ -67,6 +67,7 @@ struct KernelArgs {
 // Wavefronts of a workgroup of the exchange kernel are independent unless they form a team (no LDS, no barrier); small
 // workgroups dispatch and retire at a finer grain (2 measured best of 1..16 on launches that queue).
 constexpr int kWavesPerBlock = 2;
+constexpr int kMaxWavesPerBlock = 4;       // ... four when the whole launch is resident at once
 constexpr int kResidentWavefronts = 4096;  // 256 CUs x 4 SIMDs x 4 wavefronts: what runs at once
 
 // streams one direction of a launch serves: one per (local rank, channel, peer)
