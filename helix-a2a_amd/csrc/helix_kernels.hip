@@ -39,7 +39,12 @@
 // each other without gaps from line 0 of the entry, so a wavefront walks a
 // run as one flat sequence of 16-byte units, in passes of up to six units per
 // lane, regardless of message boundaries. All loads of a pass are issued
-// before its first store.
+// before its first store, and loads return in the order they were issued, so
+// the store of a wave access goes as soon as the loads of that access are back.
+// What a pass holds of the second, small field (the statistics at the end of
+// every message) is fetched by one load per pass and handed to the lanes that
+// store it, not by one sparse load per wave access: the load pipeline charges
+// per instruction, whatever the number of live lanes.
 //
 // Every global access goes through a buffer descriptor that spans exactly the
 // tensor it belongs to (for FIFO lines: the stream's slots, first quarter of
@@ -462,6 +467,13 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
 // ---------------------------------------------------------------------------
 // receiver
 // ---------------------------------------------------------------------------
+// A receiver's step goes to its own counter and, for part 0, to the tail in the sender's block: one store
+// instruction, lane 0 writing the one and lane 1 the other (a store costs the same with one live lane or two).
+__device__ __forceinline__ void publish_receiver_step(int64_t* mine, int64_t* senderTail, int64_t step, int lane) {
+  int64_t* target = lane == 0 ? mine : senderTail;
+  if (lane < 2 && target != nullptr) st_counter(target, step);
+}
+
 // Part `part` of the wavefronts that receive stream (s -> r, ch). It waits for the token of the sending
 // part (that part's counter beyond the step: all its lines of the step are in memory), reads its slice
 // in passes of kUnitsInFlight units per lane and stores the payload. Line flags are still compared: one
@@ -521,10 +533,7 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
         // the lines of the previous entry have been consumed (csrc/helix_alltoall.cu:427-449);
         // part 0's counter is the tail the sender's back-pressure reads
         step += 1;
-        if (lane == 0) {
-          st_counter(mine, step);
-          if (counterPart == 0) st_counter(&senderInfo[1], step);
-        }
+        publish_receiver_step(mine, counterPart == 0 ? &senderInfo[1] : nullptr, step, lane);
       }
       if (head <= step) {
         SpinGuard guard(a.spinLimitTicks, broken_word(a));
@@ -676,10 +685,7 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
   HELIX_MARK(wave, 2, false);
   if (kTeam) team_barrier();  // every wavefront of the team has the lines of the last entry in registers
   if (kTeam && leader && team_is_bad(lds)) return;
-  if (leader && lane == 0) {  // close the last entry (csrc/helix_alltoall.cu:468-472)
-    st_counter(mine, step + 1);
-    if (counterPart == 0) st_counter(&senderInfo[1], step + 1);
-  }
+  if (leader) publish_receiver_step(mine, counterPart == 0 ? &senderInfo[1] : nullptr, step + 1, lane);  // close the last entry (csrc/helix_alltoall.cu:468-472)
   HELIX_MARK(wave, 3, true);
 }
 
