@@ -467,13 +467,6 @@ __device__ __forceinline__ void run_sender(const KernelArgs& a, int s, int r, in
 // ---------------------------------------------------------------------------
 // receiver
 // ---------------------------------------------------------------------------
-// A receiver's step goes to its own counter and, for part 0, to the tail in the sender's block: one store
-// instruction, lane 0 writing the one and lane 1 the other (a store costs the same with one live lane or two).
-__device__ __forceinline__ void publish_receiver_step(int64_t* mine, int64_t* senderTail, int64_t step, int lane) {
-  int64_t* target = lane == 0 ? mine : senderTail;
-  if (lane < 2 && target != nullptr) st_counter(target, step);
-}
-
 // Part `part` of the wavefronts that receive stream (s -> r, ch). It waits for the token of the sending
 // part (that part's counter beyond the step: all its lines of the step are in memory), reads its slice
 // in passes of kUnitsInFlight units per lane and stores the payload. Line flags are still compared: one
@@ -533,7 +526,10 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
         // the lines of the previous entry have been consumed (csrc/helix_alltoall.cu:427-449);
         // part 0's counter is the tail the sender's back-pressure reads
         step += 1;
-        publish_receiver_step(mine, counterPart == 0 ? &senderInfo[1] : nullptr, step, lane);
+        if (lane == 0) {
+          st_counter(mine, step);
+          if (counterPart == 0) st_counter(&senderInfo[1], step);
+        }
       }
       if (head <= step) {
         SpinGuard guard(a.spinLimitTicks, broken_word(a));
@@ -685,7 +681,10 @@ __device__ __forceinline__ void run_receiver(const KernelArgs& a, int r, int s, 
   HELIX_MARK(wave, 2, false);
   if (kTeam) team_barrier();  // every wavefront of the team has the lines of the last entry in registers
   if (kTeam && leader && team_is_bad(lds)) return;
-  if (leader) publish_receiver_step(mine, counterPart == 0 ? &senderInfo[1] : nullptr, step + 1, lane);  // close the last entry (csrc/helix_alltoall.cu:468-472)
+  if (leader && lane == 0) {  // close the last entry (csrc/helix_alltoall.cu:468-472)
+    st_counter(mine, step + 1);
+    if (counterPart == 0) st_counter(&senderInfo[1], step + 1);
+  }
   HELIX_MARK(wave, 3, true);
 }
 
