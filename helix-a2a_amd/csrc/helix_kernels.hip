@@ -867,7 +867,8 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
   cx.positionBytes = a.positionBytes;
   cx.positionMask = a.positionMask;
   __amdgpu_buffer_rsrc_t outRsrc = make_rsrc(a.rank[r].recv0, a.recvBytes0);
-  __amdgpu_buffer_rsrc_t lseRsrc = make_rsrc(a.rank[r].recv1, a.rank[r].recv1 ? a.recvBytes1 : 0u);
+  const bool wantLse = a.rank[r].recv1 != nullptr;
+  __amdgpu_buffer_rsrc_t lseRsrc = make_rsrc(a.rank[r].recv1, wantLse ? a.recvBytes1 : 0u);
   const unsigned long long lanesUpToMe = (2ull << lane) - 1ull;  // lanes 0..lane
   const uint32_t piecesPerHead = static_cast<uint32_t>(a.headDim) / 4u;
 
@@ -1015,10 +1016,12 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
         // (senders beyond cpSize get weight 0: their pieces are read as zeros, and 0 * 0 stays 0)
         if (inSlot) lds.weight[part][slotSafe][q] = e * __builtin_amdgcn_rcpf(fmaxf(total, 1e-10f));
         // one lane per slot reports the head's combined log-sum-exp
-        const float combinedLse = fast_log(total) + m;
-        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(a.lseBase2 ? combinedLse * 1.4426950408889634f : combinedLse), lseRsrc,
-                                              (serving && q == 0) ? (slotEntry * a.heads + h) * 4u : kOutOfRange, 0,
-                                              kAuxNone);
+        if (wantLse) {  // wave-uniform: a store that every lane opts out of still costs its place in the store queue
+          const float combinedLse = fast_log(total) + m;
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(a.lseBase2 ? combinedLse * 1.4426950408889634f : combinedLse), lseRsrc,
+                                                (serving && q == 0) ? (slotEntry * a.heads + h) * 4u : kOutOfRange, 0,
+                                                kAuxNone);
+        }
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
