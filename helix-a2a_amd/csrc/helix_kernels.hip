@@ -909,7 +909,6 @@ __device__ __forceinline__ void run_combine_receiver(const KernelArgs& a, int r,
       // memory, never newer (see run_receiver). Measured on MI355X: c4 71.9 -> 70.8 us, c5a 79.5 -> 78.5; launches
       // of single-pass runs lose by it (c3 20.9 -> 21.7 us) and go straight to the vector loads.
       bool allClosed = a.longRuns != 0;
-#pragma unroll 4
       for (int q = 0; allClosed && q < a.cpSize; ++q) {
         const uint8_t* senderRow = a.workspace + static_cast<uint64_t>(q) * a.rowStrideBytes;
         const int64_t* tok = reinterpret_cast<const int64_t*>(senderRow + sender_info_offset(a.cpSize, a.maxChannels, r, ch));
