@@ -40,12 +40,12 @@ MIN_ROOFLINE_STEPS = 200
 # <kernel>_<workload>.md hold the runs these come from. These counters sit between L2 and fabric:
 # they do not tell whether the memory-side cache or DRAM served a request.
 MEASURED_TRAFFIC_BYTES = {
-    ("helix_exchange_kernel", "c3", 128): 151_137_436,   # profiles/helix_exchange_kernel_c3.md
-    ("helix_exchange_kernel", "c4", 128): 567_549_592,   # profiles/helix_exchange_kernel_c4.md
-    ("helix_exchange_kernel", "c5a", 64): 588_268_899,   # profiles/helix_exchange_kernel_c5a.md
-    ("helix_combine_kernel", "c3", 128): 118_658_125,   # profiles/helix_combine_kernel_c3.md
-    ("helix_combine_kernel", "c4", 128): 450_075_420,   # profiles/helix_combine_kernel_c4.md
-    ("helix_combine_kernel", "c5a", 64): 462_152_573,   # profiles/helix_combine_kernel_c5a.md
+    ("helix_exchange_kernel", "c3", 128): 151_117_050,   # profiles/helix_exchange_kernel_c3.md
+    ("helix_exchange_kernel", "c4", 128): 567_572_388,   # profiles/helix_exchange_kernel_c4.md
+    ("helix_exchange_kernel", "c5a", 64): 588_258_788,   # profiles/helix_exchange_kernel_c5a.md
+    ("helix_combine_kernel", "c3", 128): 118_652_719,   # profiles/helix_combine_kernel_c3.md
+    ("helix_combine_kernel", "c4", 128): 449_916_395,   # profiles/helix_combine_kernel_c4.md
+    ("helix_combine_kernel", "c5a", 64): 461_762_297,   # profiles/helix_combine_kernel_c5a.md
 }
 
 
