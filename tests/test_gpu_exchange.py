@@ -1063,13 +1063,16 @@ def test_receivers_overlapping_their_senders(hx, ops, channels):
 # graph capture
 # ---------------------------------------------------------------------------
 
-def test_exchange_and_combine_replay_from_a_captured_graph(hx, ops):
+@pytest.mark.parametrize("name", ["c2", "c4"])
+def test_exchange_and_combine_replay_from_a_captured_graph(hx, ops, name):
     # The FIFO step counters live in the workspace, not in the kernel arguments, so a captured
     # launch can be replayed: every replay walks on to the next FIFO entry. Replays are interleaved
-    # with eager work and synchronisations, and every one of them is checked.
+    # with eager work and synchronisations, and every one of them is checked. c2: single-pass runs;
+    # c4: long runs, whose wavefronts read every counter they start from -- their own and, at first,
+    # their sender's -- through the scalar cache, which must not hold what the kernel before left there.
     from helix_workloads import WORKLOADS, make_inputs
 
-    w = WORKLOADS["c2"]
+    w = WORKLOADS[name]
     ws = get_workspace(hx, w.cp)
     ins_o, ins_s = make_inputs(w, "cuda")
     plan = ops.LoopbackPlan(ins_o, ins_s, ws)
